@@ -1,0 +1,477 @@
+// Kernels of layers that mix a sequence through a short convolution and windowed attention, with fp32 arithmetic
+// wherever a norm, a score, a softmax weight or the residual stream is formed:
+//
+//   scalar_norm            x / sqrt(mean(x^2) + eps) * g with ONE gain for the row
+//   scalar_norm_residual   residual(fp32) += norm(y) * g_post ; out = norm(residual) * g_next     (one launch)
+//   poly_norm              c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3,  N(u) = u / sqrt(mean(u^2) + eps)
+//   conv_norm_cache        causal per-channel convolution over time of a fused [q | k | v | ..] projection (history
+//                          from the chunk itself or from a per-request state slot), per-head RMS norm of q and k,
+//                          value mixing, k / v into row caches, q out
+//   conv_state_update      the last taps-1 projected rows of every sequence into its state slot
+//   window_bias_attention  attention over row caches [blocks, Hkv, block, D] / [.., Dv]: causal window that keeps
+//                          the first keys, score cap, logarithmic distance bias, sink in the denominator, sigmoid
+//                          gate on the output; one wave per (token, query head), online softmax in fp32
+//
+// Element types: bf16 / fp16 / fp32 for activations and caches (fp32: the model runs entirely in 32-bit).
+#include "common.h"
+#include <math.h>
+#include <type_traits>
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
+
+// ------------------------------------------------------------------------------------------------ norms
+template <typename TI, typename TO>
+__global__ void scalar_norm_kernel(TO* __restrict__ out, const TI* __restrict__ x, const float* __restrict__ gain,
+                                   float eps, int H, long x_stride) {
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const TI* xr = x + row * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) { const float f = ldf(xr + i); ss += f * f; }
+  ss = block_sum(ss, red);
+  const float inv = (1.0f / sqrtf(ss / (float)H + eps)) * gain[0];
+  TO* orow = out + row * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) stf(orow + i, ldf(xr + i) * inv);
+}
+
+// residual += y / rms(y) * g_post ; out = residual / rms(residual) * g_next (skipped when out == nullptr)
+template <typename TY, typename TO>
+__global__ void scalar_norm_residual_kernel(TO* __restrict__ out, const TY* __restrict__ y, float* __restrict__ residual,
+                                            const float* __restrict__ g_post, const float* __restrict__ g_next,
+                                            float eps, int H, long y_stride) {
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const TY* yr = y + row * y_stride;
+  float* rr = residual + row * (long)H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) { const float f = ldf(yr + i); ss += f * f; }
+  ss = block_sum(ss, red);
+  const float inv = (1.0f / sqrtf(ss / (float)H + eps)) * g_post[0];
+  float s2 = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float r = rr[i] + ldf(yr + i) * inv;
+    rr[i] = r;
+    s2 += r * r;
+  }
+  if (out == nullptr) return;
+  s2 = block_sum(s2, red);
+  const float inv2 = (1.0f / sqrtf(s2 / (float)H + eps)) * g_next[0];
+  TO* orow = out + row * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) stf(orow + i, rr[i] * inv2);      // (each thread rereads its own stores)
+}
+
+template <typename T>
+__global__ void poly_norm_kernel(T* __restrict__ out, const T* __restrict__ z, const float* __restrict__ coef,
+                                 float eps, int F, long z_stride) {
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const T* zr = z + row * z_stride;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+    const float f = ldf(zr + i), f2 = f * f, f3 = f2 * f;
+    s2 += f2; s4 += f2 * f2; s6 += f3 * f3;
+  }
+  s2 = block_sum(s2, red);
+  s4 = block_sum(s4, red);
+  s6 = block_sum(s6, red);
+  const float n = (float)F;
+  const float a = coef[0] / sqrtf(s2 / n + eps), b = coef[1] / sqrtf(s4 / n + eps), c = coef[2] / sqrtf(s6 / n + eps);
+  const float e = coef[3];
+  T* orow = out + row * (long)F;
+  for (int i = threadIdx.x; i < F; i += blockDim.x) {
+    const float f = ldf(zr + i), f2 = f * f;
+    stf(orow + i, a * f + b * f2 + c * f2 * f + e);
+  }
+}
+
+// ---------------------------------------------------------------------------- convolution + norm + cache write
+constexpr int CONV_MAX_TAPS = 8;
+constexpr int UNIT_MAX_PER_LANE = 8;        // a head is at most 64 * 8 = 512 channels wide
+
+struct ConvArgs {
+  const void* x; long x_stride;             // [T, x_stride]: [q | k | v | ...]
+  const void* conv_w;                       // [C, taps]
+  void* state;                              // [slots, R, C], R = max(taps - 1, 1)
+  const int* slots;                         // [B]
+  const int* qsl;                           // [B + 1]
+  const int* seq_lens;                      // [B]
+  const int* token_seq;                     // [T] or null (token t is sequence t)
+  const int* positions;                     // [T]
+  const float* q_norm; const float* k_norm; // [D]
+  const float* v_first;                     // [T, G * Dv] fp32 or null
+  const float* v_lambda;                    // [1] or null
+  float* v_keep;                            // [T, G * Dv] fp32 or null
+  void* q_out;                              // [T, H, D]
+  void* k_cache; void* v_cache;             // [blocks, G, bs, D | Dv] or null
+  const int* slot_mapping;                  // [T]
+  int T, H, G, D, Dv, taps, block_size;
+  float eps;
+};
+
+template <typename T>
+__global__ void conv_norm_cache_kernel(ConvArgs a) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int s = a.token_seq ? a.token_seq[t] : t;
+  const int n = a.qsl[s + 1] - a.qsl[s];
+  const int pos = a.positions[t];
+  const int chunk_start = a.seq_lens[s] - n;
+  const int R = a.taps - 1;
+  const int C = a.H * a.D + a.G * (a.D + a.Dv);
+  const T* x = (const T*)a.x;
+  const T* w = (const T*)a.conv_w;
+  T* st = (T*)a.state + (long)a.slots[s] * (R > 0 ? R : 1) * C;
+  const bool own_state = (n == 1) && R > 0;       // the only row of its sequence: this block also moves the state on
+  const int slot = a.slot_mapping[t];
+  const int units = a.H + 2 * a.G;
+  for (int u = wave; u < units; u += nwaves) {
+    int c0, width, kind, head;                    // kind 0 q, 1 k, 2 v
+    if (u < a.H) { kind = 0; head = u; width = a.D; c0 = u * a.D; }
+    else if (u < a.H + a.G) { kind = 1; head = u - a.H; width = a.D; c0 = a.H * a.D + head * a.D; }
+    else { kind = 2; head = u - a.H - a.G; width = a.Dv; c0 = (a.H + a.G) * a.D + head * a.Dv; }
+    float acc[UNIT_MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+      const int cl = lane + it * 64;
+      acc[it] = 0.f;
+      if (cl < width) {
+        const int c = c0 + cl;
+        float hist[CONV_MAX_TAPS];                // hist[j] = input at position pos - (taps - 1 - j)
+        float v = 0.f;
+        for (int j = 0; j < a.taps; ++j) {
+          const int back = a.taps - 1 - j;
+          const int p = pos - back;
+          float uv = 0.f;
+          if (p >= chunk_start && p >= 0) uv = ldf(x + (long)(t - back) * a.x_stride + c);
+          else if (p >= 0) uv = ldf(st + (long)(R - (chunk_start - p)) * C + c);
+          hist[j] = uv;
+          v += ldf(w + (long)c * a.taps + j) * uv;
+        }
+        if (own_state) {
+          for (int k = 0; k < R; ++k) stf(st + (long)k * C + c, hist[k + 1]);
+        }
+        acc[it] = v;
+        ss += v * v;
+      }
+    }
+    if (kind < 2) {
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)width + a.eps);
+      const float* nw = kind == 0 ? a.q_norm : a.k_norm;
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) acc[it] = acc[it] * inv * nw[cl];
+      }
+    }
+    if (kind == 0) {
+      T* q = (T*)a.q_out + ((long)t * a.H + head) * a.D;
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) stf(q + cl, acc[it]);
+      }
+      continue;
+    }
+    if (kind == 2) {
+      const long vrow = (long)t * a.G * a.Dv + (long)head * a.Dv;
+      const float lam = a.v_first ? a.v_lambda[0] : 0.f;
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) {
+          if (a.v_keep) a.v_keep[vrow + cl] = acc[it];
+          if (a.v_first) acc[it] = (1.0f - lam) * acc[it] + lam * a.v_first[vrow + cl];
+        }
+      }
+    }
+    if (slot < 0 || a.k_cache == nullptr) continue;
+    const long blk = slot / a.block_size, off = slot % a.block_size;
+    T* dst = (kind == 1 ? (T*)a.k_cache : (T*)a.v_cache) + ((blk * a.G + head) * a.block_size + off) * (long)width;
+#pragma unroll
+    for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+      const int cl = lane + it * 64;
+      if (cl < width) stf(dst + cl, acc[it]);
+    }
+  }
+}
+
+// Sequences that ran two or more rows: their slot takes the last R inputs of (old state ++ this step's rows).
+// One thread per (sequence, channel) reads all R before it writes any.
+template <typename T>
+__global__ void conv_state_update_kernel(const T* __restrict__ x, long x_stride, T* __restrict__ state,
+                                         const int* __restrict__ slots, const int* __restrict__ qsl, int C, int R) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int q0 = qsl[s], n = qsl[s + 1] - q0;
+  if (c >= C || n < 2) return;
+  T* st = state + (long)slots[s] * R * C;
+  float keep[CONV_MAX_TAPS];
+  for (int k = 0; k < R; ++k) {
+    const int i = n - R + k;
+    keep[k] = i >= 0 ? ldf(x + (long)(q0 + i) * x_stride + c) : ldf(st + (long)(k + n) * C + c);
+  }
+  for (int k = 0; k < R; ++k) stf(st + (long)k * C + c, keep[k]);
+}
+
+// ------------------------------------------------------------------------------------------- attention
+struct AttnArgs {
+  const void* q;                    // [T, H, D]
+  const void* k_cache; const void* v_cache;
+  const int* block_table; long bt_stride;
+  const int* token_seq;             // [T] or null
+  const int* positions;             // [T]
+  const float* bias_scale; const float* bias_rate; const float* sinks;    // [H] or null
+  const void* gate; long gate_stride;                                      // [T, gate_stride] raw, or null
+  void* out;                        // [T, H, Dv]
+  int T, H, G, D, Dv, block_size, window, keep_first;
+  float scale, softcap;
+};
+
+template <typename T, bool VEC> struct RowDot;
+template <bool VEC> struct RowDot<float, VEC> {
+  static __device__ __forceinline__ float run(const float* k, const float* q, int D) {
+    float s = 0.f;
+    if (VEC) {
+      for (int d = 0; d < D; d += 4) {
+        const f32x4 kv = *reinterpret_cast<const f32x4*>(k + d);
+        s += kv[0] * q[d] + kv[1] * q[d + 1] + kv[2] * q[d + 2] + kv[3] * q[d + 3];
+      }
+    } else {
+      for (int d = 0; d < D; ++d) s += k[d] * q[d];
+    }
+    return s;
+  }
+};
+template <typename T, bool VEC> struct RowDot {
+  static __device__ __forceinline__ float run(const T* k, const float* q, int D) {
+    float s = 0.f;
+    if (VEC) {
+      for (int d = 0; d < D; d += 8) {
+        const typename Vec8<T>::type kv = ld8<T>(k + d);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += (float)kv[j] * q[d + j];
+      }
+    } else {
+      for (int d = 0; d < D; ++d) s += (float)k[d] * q[d];
+    }
+    return s;
+  }
+};
+
+constexpr int ATTN_MAX_WAVES = 16;
+constexpr int ATTN_V_PER_LANE = 8;          // Dv <= 512
+
+// grid (T, G, head chunks); block = waves x 64: wave w of chunk z is query head g * (H / G) + z * waves + w.
+// LDS: per wave D floats of q, 64 weights, 64 value-row offsets.
+template <typename T, bool VEC>
+__global__ void window_bias_attention_kernel(AttnArgs a) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int qpg = a.H / a.G;
+  const int hl = blockIdx.z * nwaves + wave;
+  if (hl >= qpg) return;                      // (no block-wide barrier below: a wave may leave)
+  const int h = g * qpg + hl;
+  float* sq = lds + (long)wave * (a.D + 128);
+  float* sp = sq + a.D;
+  long* srow = reinterpret_cast<long*>(lds + (((long)nwaves * (a.D + 128) + 1) & ~1L)) + wave * 64;
+  const int s = a.token_seq ? a.token_seq[t] : t;
+  const int pos = a.positions[t];
+  const T* q = (const T*)a.q + ((long)t * a.H + h) * a.D;
+  for (int d = lane; d < a.D; d += 64) sq[d] = ldf(q + d);
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int nkeep = a.window > 0 ? min(a.keep_first, lo) : 0;
+  const int total = nkeep + (pos - lo + 1);
+  const float r1 = a.bias_scale ? a.bias_scale[h] : 0.f, r2 = a.bias_rate ? a.bias_rate[h] : 0.f;
+  const int* bt = a.block_table + (long)s * a.bt_stride;
+  const T* kc = (const T*)a.k_cache;
+  const T* vc = (const T*)a.v_cache;
+  // value channels: with Dv <= 32 the lanes split the keys of a tile 2 or 4 ways as well
+  const int kparts = a.Dv <= 16 ? 4 : (a.Dv <= 32 ? 2 : 1);
+  const int cw = 64 / kparts;
+  const int kp = lane / cw, cl0 = lane % cw;
+  float acc[ATTN_V_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ATTN_V_PER_LANE; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  __builtin_amdgcn_wave_barrier();
+  for (int f0 = 0; f0 < total; f0 += 64) {
+    const int f = f0 + lane;
+    float sc = -INFINITY;
+    long vrow = 0;
+    if (f < total) {
+      const int j = f < nkeep ? f : lo + (f - nkeep);
+      const long blk = bt[j / a.block_size];
+      const long row = (blk * a.G + g) * a.block_size + (j % a.block_size);
+      sc = RowDot<T, VEC>::run(kc + row * a.D, sq, a.D) * a.scale;
+      if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
+      if (a.bias_scale) sc -= r1 * log1pf(r2 * (float)(pos - j));
+      vrow = row * a.Dv;
+    }
+    const float m_new = fmaxf(m, wave_max(sc));
+    const float p = f < total ? expf(sc - m_new) : 0.f;
+    const float corr = expf(m - m_new);          // (m = -inf on the first tile: exp(-inf) = 0)
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    sp[lane] = p;
+    srow[lane] = vrow;
+    __builtin_amdgcn_wave_barrier();
+    const int cnt = min(64, total - f0);
+#pragma unroll
+    for (int i = 0; i < ATTN_V_PER_LANE; ++i) acc[i] *= corr;
+    for (int jj = kp; jj < cnt; jj += kparts) {
+      const float pj = sp[jj];
+      const T* vr = vc + srow[jj];
+#pragma unroll
+      for (int i = 0; i < ATTN_V_PER_LANE; ++i) {
+        const int c = cl0 + i * cw;
+        if (c < a.Dv) acc[i] += pj * ldf(vr + c);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (kparts > 1) {
+#pragma unroll
+    for (int i = 0; i < ATTN_V_PER_LANE; ++i) {
+      float v = acc[i];
+      for (int o = cw; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+      acc[i] = v;
+    }
+  }
+  if (a.sinks) {                                // exp(sink) joins the denominator, once, with no value
+    const float sk = a.sinks[h];
+    const float m_f = fmaxf(m, sk);
+    const float corr = expf(m - m_f);
+    l = l * corr + expf(sk - m_f);
+#pragma unroll
+    for (int i = 0; i < ATTN_V_PER_LANE; ++i) acc[i] *= corr;
+  }
+  float mul = 1.0f / l;
+  if (a.gate) {
+    const float gv = ldf((const T*)a.gate + (long)t * a.gate_stride + h);
+    mul *= 1.0f / (1.0f + expf(-gv));
+  }
+  T* o = (T*)a.out + ((long)t * a.H + h) * a.Dv;
+  if (kp == 0) {
+#pragma unroll
+    for (int i = 0; i < ATTN_V_PER_LANE; ++i) {
+      const int c = cl0 + i * cw;
+      if (c < a.Dv) stf(o + c, acc[i] * mul);
+    }
+  }
+}
+
+template <typename F> int by_dtype(int dt, F&& f) {
+  switch (dt) {
+    case DT_BF16: f((bf16_t*)nullptr); return 0;
+    case DT_F16: f((f16_t*)nullptr); return 0;
+    case DT_F32: f((float*)nullptr); return 0;
+  }
+  return 1;
+}
+
+int norm_threads(int h) { return h >= 2048 ? 512 : (h >= 512 ? 256 : 128); }
+
+}  // namespace
+
+// out[rows, H] (dtype out_dt) = x[rows, x_stride..] (dtype in_dt) normalised with one gain
+VDAMD_API int vdamd_scalar_norm(void* out, const void* x, const float* gain, float eps, int rows, int H, long x_stride,
+                                int in_dt, int out_dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0) return 1;
+  const int th = norm_threads(H);
+  int inner = 0;
+  const int rc = by_dtype(in_dt, [&](auto* ti) {
+    using TI = std::remove_pointer_t<decltype(ti)>;
+    inner = by_dtype(out_dt, [&](auto* to) {
+      using TO = std::remove_pointer_t<decltype(to)>;
+      hipLaunchKernelGGL((scalar_norm_kernel<TI, TO>), dim3(rows), dim3(th), 0, stream, (TO*)out, (const TI*)x, gain,
+                         eps, H, x_stride);
+    });
+  });
+  return rc | inner;
+}
+
+VDAMD_API int vdamd_scalar_norm_residual(void* out, const void* y, float* residual, const float* g_post,
+                                         const float* g_next, float eps, int rows, int H, long y_stride, int y_dt,
+                                         int out_dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || (out != nullptr && g_next == nullptr)) return 1;
+  const int th = norm_threads(H);
+  int inner = 0;
+  const int rc = by_dtype(y_dt, [&](auto* ty) {
+    using TY = std::remove_pointer_t<decltype(ty)>;
+    inner = by_dtype(out_dt, [&](auto* to) {
+      using TO = std::remove_pointer_t<decltype(to)>;
+      hipLaunchKernelGGL((scalar_norm_residual_kernel<TY, TO>), dim3(rows), dim3(th), 0, stream, (TO*)out,
+                         (const TY*)y, residual, g_post, g_next, eps, H, y_stride);
+    });
+  });
+  return rc | inner;
+}
+
+VDAMD_API int vdamd_poly_norm(void* out, const void* z, const float* coef, float eps, int rows, int F, long z_stride,
+                              int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (F <= 0) return 1;
+  const int th = norm_threads(F);
+  return by_dtype(dt, [&](auto* tp) {
+    using T = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((poly_norm_kernel<T>), dim3(rows), dim3(th), 0, stream, (T*)out, (const T*)z, coef, eps, F,
+                       z_stride);
+  });
+}
+
+VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* conv_w, void* state, const int* slots,
+                                    const int* qsl, const int* seq_lens, const int* token_seq, const int* positions,
+                                    const float* q_norm, const float* k_norm, const float* v_first,
+                                    const float* v_lambda, float* v_keep, void* q_out, void* k_cache, void* v_cache,
+                                    const int* slot_mapping, int T, int B, int H, int G, int D, int Dv, int taps,
+                                    int block_size, float eps, int update_multi, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (taps < 1 || taps > CONV_MAX_TAPS || D > 64 * UNIT_MAX_PER_LANE || Dv > 64 * UNIT_MAX_PER_LANE || H % G ||
+      block_size <= 0 || (v_first != nullptr && v_lambda == nullptr))
+    return 1;
+  ConvArgs a{x, x_stride, conv_w, state, slots, qsl, seq_lens, token_seq, positions, q_norm, k_norm, v_first, v_lambda,
+             v_keep, q_out, k_cache, v_cache, slot_mapping, T, H, G, D, Dv, taps, block_size, eps};
+  const int units = H + 2 * G;
+  const int waves = units >= 4 ? 4 : units;
+  const int C = H * D + G * (D + Dv), R = taps - 1;
+  return by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((conv_norm_cache_kernel<TT>), dim3(T), dim3(64 * waves), 0, stream, a);
+    if (update_multi && R > 0)
+      hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3((C + 255) / 256, B), dim3(256), 0, stream,
+                         (const TT*)x, x_stride, (TT*)state, slots, qsl, C, R);
+  });
+}
+
+VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, const void* v_cache,
+                                          const int* block_table, long bt_stride, const int* token_seq,
+                                          const int* positions, const float* bias_scale, const float* bias_rate,
+                                          const float* sinks, const void* gate, long gate_stride, void* out, int T,
+                                          int H, int G, int D, int Dv, int block_size, int window, int keep_first,
+                                          float scale, float softcap, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H % G || D <= 0 || Dv <= 0 || Dv > 64 * ATTN_V_PER_LANE || block_size <= 0 || (bias_scale && !bias_rate)) return 1;
+  AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
+             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap};
+  const int qpg = H / G;
+  const int waves = qpg < ATTN_MAX_WAVES ? qpg : ATTN_MAX_WAVES;
+  const int chunks = (qpg + waves - 1) / waves;
+  const size_t lds = (((size_t)waves * (D + 128) + 1) & ~(size_t)1) * sizeof(float) + (size_t)waves * 64 * sizeof(long);
+  if (lds > 64 * 1024) return 2;
+  const bool vec = dt == DT_F32 ? (D % 4 == 0) : (D % 8 == 0);
+  return by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    if (vec)
+      hipLaunchKernelGGL((window_bias_attention_kernel<TT, true>), dim3(T, G, chunks), dim3(64 * waves), lds, stream, a);
+    else
+      hipLaunchKernelGGL((window_bias_attention_kernel<TT, false>), dim3(T, G, chunks), dim3(64 * waves), lds, stream, a);
+  });
+}

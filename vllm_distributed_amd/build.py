@@ -26,7 +26,12 @@ BUILD = os.path.join(ROOT, "build")
 ARCH = os.environ.get("VDAMD_GPU_ARCH", "gfx950")
 
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffast-math",
-             "-fno-gpu-rdc", "-Wno-unused-result", "-DNDEBUG"]
+             "-fno-gpu-rdc", "-Wno-unused-result", "-DNDEBUG",
+             # no packed-fp32 instructions from ordinary float code
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# sources whose fp32 arithmetic is part of a model's definition (norms, scores, softmax in 32-bit): IEEE division,
+# square roots and library exp / log / tanh instead of the fast-math forms
+EXACT_MATH_SOURCES = {"seq_mix.hip"}
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-DNDEBUG"]
 
 
@@ -62,8 +67,13 @@ def _build_lib(name: str, sources: List[str], headers: List[str], compiler: str,
     if not force and os.path.exists(lib) and os.path.exists(stamp) and open(stamp).read().strip() == digest:
         return lib
     objs = [os.path.join(BUILD, name + "." + os.path.basename(s) + ".o") for s in sources]
+    def flags_for(src: str) -> List[str]:
+        if os.path.basename(src) in EXACT_MATH_SOURCES:
+            return [f for f in flags if f != "-ffast-math"]
+        return flags
+
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as ex:
-        list(ex.map(lambda so: _run([compiler] + flags + ["-c", so[0], "-o", so[1]]), zip(sources, objs)))
+        list(ex.map(lambda so: _run([compiler] + flags_for(so[0]) + ["-c", so[0], "-o", so[1]]), zip(sources, objs)))
     _run([compiler, "-shared", "-fPIC"] + ([f"--offload-arch={ARCH}"] if compiler.endswith("hipcc") else [])
          + objs + link_flags + ["-o", lib])
     with open(stamp, "w") as f:
@@ -94,14 +104,18 @@ def build_sanitized(verbose: bool = True) -> str:
     return lib
 
 
-def build(force: bool = False, verbose: bool = True) -> List[str]:
+def build(force: bool = False, verbose: bool = True, only: tuple = ("ops", "core")) -> List[str]:
+    """``only``: which libraries to build - ``ops`` (the kernel library) and / or ``core`` (the host runtime:
+    grammars, n-gram lookup), e.g. just ``ops`` for a program that runs a model and parses nothing."""
     built = []
     hip_src = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
     headers = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".inc")))
+    if "ops" not in only:
+        hip_src = []
     if hip_src:
         built.append(_build_lib("libvdamd_ops.so", hip_src, headers, _hipcc(), HIP_FLAGS, [], force))
     core_dir = os.path.join(CSRC, "core")
-    if os.path.isdir(core_dir):
+    if os.path.isdir(core_dir) and "core" in only:
         cpp = sorted(os.path.join(core_dir, f) for f in os.listdir(core_dir) if f.endswith(".cpp"))
         hdr = sorted(os.path.join(core_dir, f) for f in os.listdir(core_dir) if f.endswith(".h"))
         if cpp:

@@ -112,6 +112,20 @@ def normalize_hf_config(cfg: Dict[str, Any]) -> None:
                                      "layer_norm_eps": 1e-5, "hidden_act": "quick_gelu"}, **(cfg.get("vision_config") or {}))
         cfg.setdefault("architectures", ["LlavaNextForConditionalGeneration" if cfg["mm_model_type"] == "llava_next"
                                          else "LlavaForConditionalGeneration"])
+    if cfg.get("architecture") == "Tavulix" or cfg.get("model_type") == "tavulix":
+        # Tavulix lists its layers one by one and spells the global sizes its own way; the keys every accessor
+        # reads are derived here (heads and head size of the first layer: informational, layers may differ)
+        cfg.setdefault("model_type", "tavulix")
+        cfg.setdefault("architectures", ["TavulixForCausalLM"])
+        mixers = [l.get("mixer") or {} for l in cfg.get("layers") or []]
+        first = mixers[0] if mixers else {}
+        for k, v in (("hidden_size", cfg.get("width")), ("vocab_size", cfg.get("vocab")),
+                     ("max_position_embeddings", cfg.get("max_positions")), ("num_hidden_layers", len(mixers)),
+                     ("num_attention_heads", first.get("heads", 1)),
+                     ("num_key_value_heads", first.get("kv_heads") or first.get("heads", 1)),
+                     ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
+            if cfg.get(k) is None and v is not None:
+                cfg[k] = v
     if cfg.get("model_type") == "dbrx":
         # DBRX nests its attention and expert settings
         a, f = cfg.get("attn_config") or {}, cfg.get("ffn_config") or {}
@@ -607,6 +621,17 @@ class VllmConfig:
                 # drafts are looked up in the tokens generated so far: the scheduler cannot run ahead of them
                 logger.info("speculative decoding: async scheduling off")
                 self.scheduler_config.async_scheduling = False
+        from .models.registry import keeps_request_state
+        if keeps_request_state(mc.architecture):
+            if self.cache_config.enable_prefix_caching:
+                logger.info("%s keeps per-request layer state: prefix caching off", mc.architecture)
+                self.cache_config.enable_prefix_caching = False
+            if self.speculative_config is not None:
+                raise ValueError(f"speculative decoding is not supported for {mc.architecture}: a rejected draft "
+                                 f"would have advanced its per-request layer state")
+            if self.kv_transfer_config is not None:
+                raise ValueError(f"KV transfer is not supported for {mc.architecture}: its per-request layer state "
+                                 f"is not part of the blocks")
         if mc.num_attention_heads % pc.tensor_parallel_size != 0:
             raise ValueError(f"num_attention_heads ({mc.num_attention_heads}) must be divisible "
                              f"by tensor_parallel_size ({pc.tensor_parallel_size})")

@@ -95,7 +95,7 @@ class EngineCore:
                                    max_loras=vllm_config.lora_config.max_loras if vllm_config.lora_config else 0,
                                    speculative_config=vllm_config.speculative_config,
                                    sliding_window=None if kv_connector is not None else self.kv_window,
-                                   pipeline_depth=pp)
+                                   pipeline_depth=pp, keep_first=self.kv_keep_first)
         self.max_concurrent = max(1, self.executor.max_concurrent_batches)
         self._tune_gc()
         self.batch_queue: Deque[Tuple[object, SchedulerOutput]] = deque()
@@ -123,7 +123,9 @@ class EngineCore:
         if cc.num_gpu_blocks_override is not None:
             num_blocks = int(cc.num_gpu_blocks_override)
         else:
-            num_blocks = min(int(a // s.bytes_per_block) for a, s in zip(avail, specs))
+            seqs = self.vllm_config.scheduler_config.max_num_seqs       # (per-request layer state comes off the top)
+            num_blocks = min(int(max(a - seqs * getattr(s, "state_bytes_per_request", 0), 0) // s.bytes_per_block)
+                             for a, s in zip(avail, specs))
             # no point holding more than every sequence at full length
             cap = self.vllm_config.scheduler_config.max_num_seqs * cdiv(
                 self.vllm_config.model_config.max_model_len, cc.block_size)
@@ -138,6 +140,7 @@ class EngineCore:
         # every layer of every worker windowed: blocks that slid out of the widest window are dead
         wins = [getattr(s, "sliding_window", None) for s in specs]
         self.kv_window = max(wins) if wins and all(w is not None for w in wins) else None
+        self.kv_keep_first = max((getattr(s, "keep_first", 0) or 0) for s in specs) if specs else 0
         self.executor.initialize_from_config([KVCacheConfig(num_blocks=num_blocks)] * len(specs))
         return num_blocks
 
@@ -182,6 +185,23 @@ class EngineCore:
         self.timer.add_head(schedule=t1 - t0, execute=t2 - t1, update=t3 - t2)
         self.timer.add_step(out)
         return res
+
+    def extend_request(self, request_id: str, token_ids: List[int]) -> None:
+        self.scheduler.extend_request(request_id, token_ids)
+
+    def step_forced(self, plan: Dict[str, int], logits_wanted: Optional[Dict[str, List[int]]] = None,
+                    ) -> Tuple[List[EngineCoreOutput], Optional[ModelRunnerOutput]]:
+        """One step of exactly the given requests and token counts (``Scheduler.schedule_forced``), run to its
+        end: the replay of a recorded schedule.  Returns the step's outputs and the workers' reply, which
+        carries the logits asked for."""
+        self._check_alive()
+        if self.batch_queue:
+            raise RuntimeError("a forced step cannot overtake steps in flight")
+        so = self.scheduler.schedule_forced(plan, logits_wanted)
+        out = self.executor.execute_model(so)
+        if hasattr(out, "result"):
+            out = out.result()
+        return self.scheduler.update_from_output(so, out), out
 
     @staticmethod
     def _worth_running(so: SchedulerOutput) -> bool:

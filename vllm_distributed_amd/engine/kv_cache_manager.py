@@ -99,9 +99,11 @@ class KVCacheManager:
     WINDOW_MARGIN = 128
 
     def __init__(self, num_blocks: int, block_size: int, max_model_len: int,
-                 enable_caching: bool = True, sliding_window: Optional[int] = None):
+                 enable_caching: bool = True, sliding_window: Optional[int] = None, keep_first: int = 0):
         # every attention layer sees at most this many most recent keys (None: some layer sees all)
         self.window = int(sliding_window) if sliding_window else None
+        # ... and, besides them, the first `keep_first` keys of the sequence: the blocks over those are never released
+        self.keep_first = int(keep_first or 0)
         self.num_released: Dict[str, int] = {}       # leading blocks already given back, per request
         self.block_size = block_size
         self.max_model_len = max_model_len
@@ -220,7 +222,8 @@ class KVCacheManager:
         if not held:
             return 0
         dead = (request.num_computed_tokens - self.window - self.WINDOW_MARGIN) // self.block_size
-        done = self.num_released.get(request.request_id, 0)
+        kept = cdiv(self.keep_first, self.block_size)          # leading blocks every query keeps reading
+        done = max(self.num_released.get(request.request_id, 0), kept)
         dead = min(dead, len(held))
         if dead <= done:
             return 0

@@ -63,7 +63,7 @@ class Scheduler:
     def __init__(self, scheduler_config: SchedulerConfig, cache_config: CacheConfig,
                  num_blocks: int, include_new_token_ids: bool = True,
                  kv_connector=None, max_loras: int = 0, speculative_config=None,
-                 sliding_window: Optional[int] = None, pipeline_depth: int = 1):
+                 sliding_window: Optional[int] = None, pipeline_depth: int = 1, keep_first: int = 0):
         self.config = scheduler_config
         # pipeline parallelism keeps `pipeline_depth` batches in flight, and a stage only has work
         # while a batch is at it: the running requests are dealt out over that many micro-batches
@@ -77,7 +77,10 @@ class Scheduler:
         # a request that will sample carries a placeholder for the unknown token
         self.async_scheduling = bool(scheduler_config.async_scheduling)
         self.kv = KVCacheManager(num_blocks, cache_config.block_size, self.max_model_len,
-                                 cache_config.enable_prefix_caching, sliding_window=sliding_window)
+                                 cache_config.enable_prefix_caching, sliding_window=sliding_window,
+                                 keep_first=keep_first)
+        # token replay: tokens appended to requests the workers already hold, delivered with the next step
+        self._appended_tokens: Dict[str, List[int]] = {}
         self.requests: Dict[str, Request] = {}
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
@@ -121,7 +124,8 @@ class Scheduler:
             raise ValueError(f"duplicate request id {request.request_id}")
         if request.num_prompt_tokens == 0:
             raise ValueError("empty prompt")
-        if request.num_prompt_tokens >= self.max_model_len:
+        # (a request that samples nothing needs no position for an output token)
+        if request.num_prompt_tokens >= self.max_model_len + int(bool(request.sampling_params.score_only)):
             raise ValueError(f"prompt ({request.num_prompt_tokens} tokens) does not fit "
                              f"max_model_len ({self.max_model_len})")
         if request.lora_request is not None and self.max_loras <= 0:
@@ -374,6 +378,76 @@ class Scheduler:
         self.step_id += 1
         return out
 
+    # ---------------------------------------------------------- token replay
+    def extend_request(self, request_id: str, token_ids: List[int]) -> None:
+        """Append given tokens to a live request's prompt (a trace that arrives step by step).  Only for requests
+        that sample nothing (``SamplingParams.score_only``): a sampled token would already stand at that place."""
+        req = self.requests[request_id]
+        if not req.sampling_params.score_only or req.output_token_ids:
+            raise ValueError(f"{request_id} is not a replayed request: its prompt cannot grow")
+        if req.num_tokens + len(token_ids) > self.max_model_len:
+            raise ValueError(f"{request_id} would outgrow max_model_len ({self.max_model_len})")
+        req.prompt_token_ids.extend(token_ids)
+        req.all_token_ids.extend(token_ids)
+        req.metrics.num_prompt_tokens = len(req.prompt_token_ids)
+        if request_id in self._known_to_workers:
+            self._appended_tokens.setdefault(request_id, []).extend(token_ids)
+
+    def schedule_forced(self, plan: Dict[str, int],
+                        logits_wanted: Optional[Dict[str, List[int]]] = None) -> SchedulerOutput:
+        """A step whose composition the caller dictates: ``plan[req] = number of that request's next tokens to
+        run``, in batch order.  Requests not named sit the step out; a waiting request named here is admitted.
+        Blocks and batch rows come from the same managers as in ``schedule``; nothing is preempted - a plan
+        that does not fit the pool or the sequence limit is the caller's error."""
+        num_scheduled: Dict[str, int] = {}
+        new_reqs: List[NewRequestData] = []
+        cached = CachedRequestData()
+        now = time.time()
+        for rid, n in plan.items():
+            req = self.requests[rid]
+            if n <= 0 or req.num_computed_tokens + n > req.num_tokens:
+                raise ValueError(f"{rid}: {n} tokens asked, {req.num_tokens - req.num_computed_tokens} left to run")
+            if req.status == RequestStatus.RUNNING:
+                held = self.kv.req_blocks.get(rid)
+                if held is not None and req.num_computed_tokens + n <= len(held) * self.kv.block_size:
+                    new_blocks = _NO_BLOCKS
+                else:
+                    new_blocks = self.kv.allocate_slots(req, n)
+                    if new_blocks is None:
+                        raise RuntimeError(f"out of KV blocks for {rid} ({self.kv.num_free_blocks} free)")
+                self._add_cached(cached, req, new_blocks)
+            else:
+                if len(self.running) >= self.max_num_seqs:
+                    raise RuntimeError(f"{rid}: every one of the {self.max_num_seqs} sequence slots is taken")
+                blocks = self.kv.allocate_slots(req, n)
+                if blocks is None:
+                    raise RuntimeError(f"out of KV blocks for {rid} ({self.kv.num_free_blocks} free)")
+                self.waiting.remove(req)
+                req.status = RequestStatus.RUNNING
+                self.running.append(req)
+                if req.metrics.first_scheduled_time is None:
+                    req.metrics.first_scheduled_time = now
+                req.num_cached_tokens = 0
+                new_reqs.append(NewRequestData(
+                    req_id=rid, prompt_token_ids=list(req.prompt_token_ids), sampling_params=req.sampling_params,
+                    block_ids=blocks, num_computed_tokens=0, output_token_ids=list(req.output_token_ids),
+                    lora_request=req.lora_request, mm_inputs=req.mm_inputs))
+                self._known_to_workers.add(rid)
+                self._appended_tokens.pop(rid, None)
+            num_scheduled[rid] = n
+            req.num_computed_tokens += n
+        appended = {r: t for r, t in self._appended_tokens.items() if r in self._known_to_workers}
+        self._appended_tokens = {}
+        out = SchedulerOutput(
+            step_id=self.step_id, scheduled_new_reqs=new_reqs, scheduled_cached_reqs=cached,
+            num_scheduled_tokens=num_scheduled, total_num_scheduled_tokens=sum(num_scheduled.values()),
+            finished_req_ids=self._finished_since_last, preempted_req_ids=self._preempted_since_last,
+            appended_prompt_tokens=appended or None, logits_wanted=logits_wanted or None)
+        self._finished_since_last = set()
+        self._preempted_since_last = set()
+        self.step_id += 1
+        return out
+
     def _note_sampling(self, req: Request) -> None:
         """Async mode: if this step runs the request's last known position it will
         sample a token; account for it so the next step can be scheduled now."""
@@ -610,6 +684,7 @@ class Scheduler:
             self._known_to_workers.discard(req.request_id)
             self._finished_since_last.add(req.request_id)
         self._pending_new_tokens.pop(req.request_id, None)
+        self._appended_tokens.pop(req.request_id, None)
         self.requests.pop(req.request_id, None)
 
     # ----------------------------------------------------------------- stats

@@ -57,6 +57,10 @@ class SchedulerOutput:
     # for 1 + len(drafts) tokens
     scheduled_spec_decode_tokens: Optional[Dict[str, List[int]]] = None
     kv_connector_metadata: Optional[Any] = None
+    # token replay (``Scheduler.schedule_forced``): tokens appended to the prompt of a request the workers
+    # already hold, and, per request, the places among this step's tokens whose logits the caller wants back
+    appended_prompt_tokens: Optional[Dict[str, List[int]]] = None
+    logits_wanted: Optional[Dict[str, List[int]]] = None
 
     @property
     def is_empty(self) -> bool:
@@ -83,6 +87,8 @@ class ModelRunnerOutput:
     timing: Optional[Dict[str, float]] = None
     # req_id -> tokens the workers' draft model proposes after the request's newest token
     draft_token_ids: Optional[Dict[str, List[int]]] = None
+    # req_id -> float32 array [places, vocab]: the logits a step's caller asked for (``logits_wanted``)
+    logits: Optional[Dict[str, Any]] = None
 
 
 EMPTY_MODEL_RUNNER_OUTPUT = ModelRunnerOutput()
@@ -101,11 +107,18 @@ class KVCacheSpec:
     sliding_window: Optional[int] = None
     # bytes per block of further caches held over the same blocks (a draft model's layers)
     extra_bytes_per_block: int = 0
+    # windowed layers that also see the first tokens of the sequence: the blocks over these stay with the request
+    keep_first: int = 0
+    # cached values per token summed over the layers, when they are not ``2 x heads x head_dim`` each
+    values_per_token: Optional[int] = None
+    # bytes of per-request layer state (convolution tails, recurrences) each sequence slot takes beside the blocks
+    state_bytes_per_request: int = 0
 
     @property
     def bytes_per_block(self) -> int:
-        return (2 * self.num_layers * self.block_size * self.num_kv_heads * self.head_dim * self.dtype_bytes
-                + self.extra_bytes_per_block)
+        per_token = (self.values_per_token if self.values_per_token is not None
+                     else 2 * self.num_layers * self.num_kv_heads * self.head_dim)
+        return self.block_size * per_token * self.dtype_bytes + self.extra_bytes_per_block
 
     @property
     def bytes_per_token(self) -> int:

@@ -195,6 +195,10 @@ def build_parser() -> argparse.ArgumentParser:
     pbe.add_argument("--output-len", type=int, default=64)
     EngineArgs.add_cli_args(pbe)
     pbe.set_defaults(dispatch_function=cmd_bench)
+    from . import trace_replay
+    pr = sub.add_parser("replay-trace", help="replay a recorded schedule of token ids (stdin) and write logits")
+    trace_replay.add_args(pr)
+    pr.set_defaults(dispatch_function=trace_replay.cmd_replay)
     from . import client
     pc = sub.add_parser("chat", help="interactive chat with a running server")
     client.add_client_args(pc)

@@ -36,6 +36,9 @@ class AttentionMetadata:
     decode_workspace: Optional[torch.Tensor] = None
     # every prefill sequence of the step starts at position 0 (no cached context, no earlier chunk)
     prefill_fresh: bool = False
+    # [B] int32: the slot of each sequence in per-request state tensors (layers with recurrent or convolution
+    # state; the persistent batch's row), or None when the model keeps no such state
+    state_slots: Optional[torch.Tensor] = None
 
     def token_rows(self, positions: torch.Tensor):
         """Per token of the step: the block-table row it reads (None = its own index: a pure decode batch)
@@ -200,6 +203,66 @@ class LatentAttention(Attention):
         md = _CTX.attn_metadata
         rows, lens = md.token_rows(_CTX.positions)
         return ops.mla_attention(q, self.k_cache, self.v_cache, md.block_table, rows, lens, self.scale, md.max_seq_len)
+
+
+class WindowBiasAttention(Attention):
+    """Attention whose window keeps the first keys of the sequence, with a logarithmic distance bias instead of
+    a rotation, an optional score cap, a sink in the softmax denominator and a sigmoid gate on each head's output;
+    key and value heads may differ in size.  A query at position ``i`` sees key ``j <= i`` when
+    ``i - j < window`` or ``j < keep_first``; its score is ``cap(q.k * scale) - bias_scale[h] * ln(1 +
+    bias_rate[h] * (i - j))``.  The caches are plain rows, ``[blocks, Hkv, block, dim]`` and ``[blocks, Hkv,
+    block, vdim]``, written by ``ops.conv_norm_cache`` (this layer's callers convolve and normalise q / k / v
+    first); scores, softmax and the weighted sum of values are fp32 in every dtype."""
+    row_cache = True
+
+    def __init__(self, num_heads: int, dim: int, vdim: int, num_kv_heads: int, scale: float, layer_idx: int,
+                 window: int = 0, keep_first: int = 0, softcap: Optional[float] = None, distance_bias: bool = True,
+                 sink: bool = True):
+        super().__init__(num_heads, dim, num_kv_heads, scale, layer_idx, sliding_window=window, softcap=softcap)
+        self.vdim = vdim
+        self.keep_first = int(keep_first or 0) if self.window else 0
+        f32 = torch.float32
+        # (fp32 whatever the model dtype: they enter the scores directly)
+        self.bias_scale = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if distance_bias else None
+        self.bias_rate = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if distance_bias else None
+        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if sink else None
+
+    def kv_cache_shapes(self, num_blocks: int, block_size: int):
+        return ((num_blocks, self.num_kv_heads, block_size, self.head_dim),
+                (num_blocks, self.num_kv_heads, block_size, self.vdim))
+
+    def kv_values_per_token(self) -> int:
+        return self.num_kv_heads * (self.head_dim + self.vdim)
+
+    def forward_cached(self, q: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``q[T, Hq, dim]`` (this step's keys and values already cached), ``gate[T, Hq]`` raw -> ``[T, Hq * vdim]``."""
+        md = _CTX.attn_metadata
+        t = q.shape[0]
+        if md is None:               # memory-profiling pass: no cache bound
+            return q.new_zeros((t, self.num_heads * self.vdim))
+        rows = None if md.num_prefills == 0 else md.token_rows(_CTX.positions)[0]
+        out = ops.window_bias_attention(q, self.k_cache, self.v_cache, md.block_table, md.query_start_loc, md.seq_lens,
+                                        rows, _CTX.positions, self.scale, self.softcap, self.window, self.keep_first,
+                                        self.bias_scale, self.bias_rate, self.sink, gate, md.max_query_len)
+        return out.view(t, self.num_heads * self.vdim)
+
+
+class ScalarRMSNorm(nn.Module):
+    """RMS norm whose gain is a single number for all coordinates, in fp32 arithmetic; ``forward`` returns the
+    model dtype (the input of a projection), ``residual_add`` folds a sublayer's output into the fp32 residual
+    stream through this norm and hands back the next sublayer's normed input in the same launch."""
+
+    def __init__(self, eps: float, dtype: torch.dtype):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones((), dtype=torch.float32), requires_grad=False)
+        self.eps, self.dtype = eps, dtype
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.scalar_rms_norm(x, self.weight, self.eps, out_dtype or self.dtype)
+
+    def residual_add(self, y: torch.Tensor, residual: torch.Tensor, then: Optional["ScalarRMSNorm"] = None):
+        return ops.scalar_norm_residual(y, self.weight, residual, None if then is None else then.weight, self.eps,
+                                        self.dtype)
 
 
 class RMSNorm(nn.Module):

@@ -1,0 +1,52 @@
+"""Short causal convolutions over the columns of a fused projection, with per-request state.
+
+A layer that convolves its projections over time has to remember the last ``taps - 1`` projected rows of every
+live request: a prompt may arrive in portions, and a decoded token needs its predecessors' projections.  That
+state lives in one tensor per layer, ``[slots, taps - 1, channels]`` in the model dtype, indexed by the request's
+row in the worker's persistent batch (``AttentionMetadata.state_slots``); the model runner allocates it next to
+the KV cache.  Nothing is cleared when a row changes owner: positions before a sequence's start read as zero
+because of where they are, not because of what the slot holds.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+
+class ShortConv(nn.Module):
+    """``weight[channels, taps]`` for the leading ``channels`` columns of a fused projection; the checkpoint may
+    hold it in pieces (one per projection), loaded into consecutive row ranges."""
+
+    def __init__(self, piece_sizes: Sequence[int], taps: int, dtype: torch.dtype):
+        super().__init__()
+        self.piece_sizes = list(piece_sizes)
+        self.channels, self.taps = sum(self.piece_sizes), int(taps)
+        if self.taps < 1:
+            raise ValueError("a convolution needs at least one tap")
+        self.weight = nn.Parameter(torch.empty(self.channels, self.taps, dtype=dtype), requires_grad=False)
+        self.weight.weight_loader = self.load_piece          # type: ignore[attr-defined]
+        self.state: Optional[torch.Tensor] = None
+        self.dtype = dtype
+
+    def load_piece(self, param: nn.Parameter, w: torch.Tensor, shard_id: Optional[int] = None) -> None:
+        from ..utils import materialize
+        w = materialize(w)
+        if shard_id is None:
+            assert tuple(w.shape) == tuple(param.shape), (w.shape, param.shape)
+            param.data.copy_(w)
+            return
+        off, n = sum(self.piece_sizes[:shard_id]), self.piece_sizes[shard_id]
+        assert tuple(w.shape) == (n, self.taps), (w.shape, n, self.taps)
+        param.data[off:off + n].copy_(w)
+
+    # ---- per-request state, owned by the model runner
+    def state_shape(self, num_slots: int) -> Tuple[int, int, int]:
+        return (num_slots, max(self.taps - 1, 1), self.channels)
+
+    def state_values_per_slot(self) -> int:
+        return max(self.taps - 1, 1) * self.channels
+
+    def bind_state(self, state: Optional[torch.Tensor]) -> None:
+        self.state = state

@@ -48,6 +48,9 @@ def hf_weight_shapes(mc: ModelConfig) -> Dict[str, Tuple[int, ...]]:
 
 
 def _weight_shapes(c: dict, arch: str) -> Dict[str, Tuple[int, ...]]:
+    if arch in ("TavulixForCausalLM", "Tavulix"):
+        from .tavulix import weight_shapes
+        return weight_shapes(c)
     if arch == "MedusaModel":
         h = c["hidden_size"]
         out = {}
@@ -449,6 +452,10 @@ def dummy_weights_iterator(mc: ModelConfig, device: torch.device,
         if want is not None and not want(name):
             continue
         gen.manual_seed(_seed_for(name, mc.seed))
+        if mc.architecture in ("TavulixForCausalLM", "Tavulix"):
+            from .tavulix import random_weight
+            yield name, random_weight(name, shape, gen, device, dtype)
+            continue
         if awq and _QUANTIZED_LINEAR.search(name) and shape[1] % g == 0 and shape[0] % 8 == 0:
             out_f, in_f = shape
             base = name[:-len(".weight")]

@@ -64,6 +64,9 @@ _MODELS: Dict[str, Tuple[str, str]] = {
     "GraniteMoeSharedForCausalLM": ("mixtral", "GraniteMoeSharedForCausalLM"),
     "LlavaForConditionalGeneration": ("llava", "LlavaForConditionalGeneration"),
     "LlavaNextForConditionalGeneration": ("llava", "LlavaNextForConditionalGeneration"),
+    # learned positions, convolved q / k / v, windowed attention with kept first keys, PolyNorm feed-forward
+    "TavulixForCausalLM": ("tavulix", "TavulixForCausalLM"),
+    "Tavulix": ("tavulix", "TavulixForCausalLM"),
     # draft heads of speculative decoding (never a served model by themselves; worker/draft_model.py)
     "EagleLlamaForCausalLM": ("spec_heads", "EagleLlamaForCausalLM"),
     "Eagle3LlamaForCausalLM": ("spec_heads", "Eagle3LlamaForCausalLM"),
@@ -71,6 +74,15 @@ _MODELS: Dict[str, Tuple[str, str]] = {
     "DeepSeekMTP": ("spec_heads", "DeepSeekMTP"),
     "MedusaModel": ("spec_heads", "MedusaModel"),
 }
+
+
+# architectures whose layers keep per-request state besides the KV cache (convolution tails, recurrences): a cached
+# prefix's blocks do not bring that state back, so prefix reuse is off for them
+_KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix"}
+
+
+def keeps_request_state(arch: str) -> bool:
+    return arch in _KEEPS_REQUEST_STATE
 
 
 def register_model(arch: str, module: str, cls: str) -> None:

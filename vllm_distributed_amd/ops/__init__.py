@@ -261,6 +261,15 @@ def linear(x, weight, bias=None, out=None):
     return torch.nn.functional.linear(x, weight, bias)
 
 
+def linear_f32(x, weight):
+    """``x @ weight^T`` with the fp32 accumulators kept as the result (logits that are post-processed in fp32)."""
+    if x.dtype == torch.float32:
+        return torch.nn.functional.linear(x, weight)
+    if x.is_cuda and x.dim() == 2:
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    return torch.nn.functional.linear(x.float(), weight.float())
+
+
 _GELU_KINDS = {"gelu": "none", "gelu_new": "tanh", "gelu_pytorch_tanh": "tanh", "gelu_fast": "tanh",
                "gelu_tanh": "tanh"}
 
@@ -605,3 +614,54 @@ def mla_prep_ok(x: torch.Tensor) -> bool:
 
 def mla_prep(q, nope, q_lat, latent, norm_weight, eps, cos_sin, positions, k_cache, v_cache, slot_mapping):
     return _hip.mla_prep(q, nope, q_lat, latent, norm_weight, eps, cos_sin, positions, k_cache, v_cache, slot_mapping)
+
+
+# ------------------------------------------------ single-gain norms, PolyNorm, convolved q/k/v, windowed attention
+def scalar_rms_norm(x, gain, eps: float, out_dtype):
+    """RMS norm with one gain for the whole row (fp32 arithmetic), result in ``out_dtype``."""
+    if _use_hip(x):
+        return _hip.scalar_rms_norm(x, gain, eps, out_dtype)
+    return torch_ref.scalar_rms_norm(x, gain, eps, out_dtype)
+
+
+def scalar_norm_residual(y, post_gain, residual, next_gain, eps: float, out_dtype):
+    """``residual += norm(y) * post_gain`` on the fp32 residual stream, and (with ``next_gain``) the normed input of
+    the next sublayer in ``out_dtype``: one launch."""
+    if _use_hip(y):
+        return _hip.scalar_norm_residual(y, post_gain, residual, next_gain, eps, out_dtype)
+    return torch_ref.scalar_norm_residual(y, post_gain, residual, next_gain, eps, out_dtype)
+
+
+def poly_norm(z, coef, eps: float):
+    if _use_hip(z):
+        return _hip.poly_norm(z, coef, eps)
+    return torch_ref.poly_norm(z, coef, eps)
+
+
+def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
+                    num_kv_heads: int, dim: int, vdim: int, q_norm, k_norm, eps: float, v_first, v_lambda,
+                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
+    """Short convolution (with per-request state) + per-head q / k norm + value mixing + cache write over a fused
+    projection; see ``torch_ref.conv_norm_cache``.  ``token_seq`` (None: row ``t`` belongs to sequence ``t``) and
+    ``positions`` tell the kernel which sequence and position each row has."""
+    if _use_hip(x):
+        return _hip.conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
+                                    num_heads, num_kv_heads, dim, vdim, q_norm, k_norm, eps, v_first, v_lambda,
+                                    keep_v, k_cache, v_cache, slot_mapping, has_prefill)
+    return torch_ref.conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, num_heads,
+                                     num_kv_heads, dim, vdim, q_norm, k_norm, eps, v_first, v_lambda, keep_v,
+                                     k_cache, v_cache, slot_mapping)
+
+
+def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
+                          scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
+                          gate, max_query_len: int = 0):
+    """Attention over row caches with a window that keeps the first keys, a logarithmic distance bias, a sink in
+    the denominator and an output gate; see ``torch_ref.window_bias_attention``."""
+    if _use_hip(q):
+        attention_calls["hip"] += 1
+        return _hip.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq,
+                                          positions, scale, softcap, window, keep_first, bias_scale, bias_rate, sinks,
+                                          gate, max_query_len)
+    return torch_ref.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, scale,
+                                           softcap, window, keep_first, bias_scale, bias_rate, sinks, gate)

@@ -64,6 +64,11 @@ def load() -> ctypes.CDLL:
         "vdamd_fp4a16_gemm": [P, L, P, L, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_fp4_dequant": [P, P, P, P, I, I, I, P],
         "vdamd_fp4a16_gemm_grouped": [P, L, P, L, P, P, L, L, P, P, I, I, I, I, I, P],
+        "vdamd_scalar_norm": [P, P, P, F, I, I, L, I, I, P],
+        "vdamd_scalar_norm_residual": [P, P, P, P, P, F, I, I, L, I, I, P],
+        "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
+        "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, I, P],
+        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, L, P] + [I] * 8 + [F, F, I, P],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -1199,4 +1204,129 @@ def mla_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: torch.Tens
                                None if slot_mapping is None else v_cache.data_ptr(),
                                None if slot_mapping is None else slot_mapping.data_ptr(), t, h, rank, rope, bs,
                                _dt(q), fp8, _stream()), "mla_prep")
+    return out
+
+
+# ------------------------------------------------ single-gain norms, PolyNorm, convolved q/k/v, windowed attention
+def _i32(t: Optional[torch.Tensor], name: str) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    assert t.dtype == torch.int32 and t.is_contiguous() and t.is_cuda, f"{name}: int32 contiguous device tensor expected"
+    return t
+
+
+def _f32_vec(t: Optional[torch.Tensor], n: int, name: str) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    assert t.dtype == torch.float32 and t.is_cuda and t.numel() == n and t.is_contiguous(), \
+        f"{name}: {n} contiguous fp32 values expected, got {tuple(t.shape)} {t.dtype}"
+    return t
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def scalar_rms_norm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    h = x.shape[-1]
+    x2 = x.reshape(-1, h)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    out = torch.empty((x2.shape[0], h), dtype=out_dtype, device=x.device)
+    _check(_LIB.vdamd_scalar_norm(out.data_ptr(), x2.data_ptr(), _f32_vec(gain, 1, "gain").data_ptr(), float(eps),
+                                  x2.shape[0], h, x2.stride(0), _dt(x2), _dt(out), _stream()), "scalar_norm")
+    return out.view(x.shape[:-1] + (h,))
+
+
+def scalar_norm_residual(y: torch.Tensor, post_gain: torch.Tensor, residual: torch.Tensor,
+                         next_gain: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype):
+    t, h = y.shape
+    assert residual.shape == (t, h) and residual.dtype == torch.float32 and residual.is_contiguous() and y.stride(1) == 1
+    out = torch.empty((t, h), dtype=out_dtype, device=y.device) if next_gain is not None else None
+    _check(_LIB.vdamd_scalar_norm_residual(
+        _ptr(out), y.data_ptr(), residual.data_ptr(), _f32_vec(post_gain, 1, "post_gain").data_ptr(),
+        _ptr(_f32_vec(next_gain, 1, "next_gain")), float(eps), t, h, y.stride(0), _dt(y),
+        _DT[out_dtype], _stream()), "scalar_norm_residual")
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    f = z.shape[-1]
+    z2 = z.reshape(-1, f)
+    if z2.stride(-1) != 1:
+        z2 = z2.contiguous()
+    out = torch.empty((z2.shape[0], f), dtype=z.dtype, device=z.device)
+    _check(_LIB.vdamd_poly_norm(out.data_ptr(), z2.data_ptr(), _f32_vec(coef, 4, "coef").data_ptr(), float(eps),
+                                z2.shape[0], f, z2.stride(0), _dt(z2), _stream()), "poly_norm")
+    return out.view(z.shape)
+
+
+CONV_MAX_TAPS = 8
+UNIT_MAX_WIDTH = 512
+
+
+def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
+                    num_kv_heads: int, dim: int, vdim: int, q_norm, k_norm, eps: float, v_first, v_lambda,
+                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
+    t = x.shape[0]
+    c = num_heads * dim + num_kv_heads * (dim + vdim)
+    taps = conv_weight.shape[1]
+    r = max(taps - 1, 1)
+    b = seq_lens.shape[0]
+    assert x.dim() == 2 and x.shape[1] >= c and x.stride(1) == 1 and x.is_cuda
+    assert conv_weight.shape == (c, taps) and conv_weight.dtype == x.dtype and conv_weight.is_contiguous()
+    assert 1 <= taps <= CONV_MAX_TAPS and dim <= UNIT_MAX_WIDTH and vdim <= UNIT_MAX_WIDTH
+    assert state is not None and state.dtype == x.dtype and state.is_contiguous() and state.shape[1:] == (r, c), \
+        (None if state is None else state.shape, (r, c))
+    assert slots.shape[0] == b and query_start_loc.shape[0] >= b + 1 and positions.shape[0] >= t
+    assert slot_mapping.shape[0] >= t and (token_seq is None or token_seq.shape[0] >= t)
+    assert token_seq is not None or t <= b, "rows without a sequence"
+    if slots.dtype != torch.int32:
+        slots = slots.to(torch.int32)
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        assert k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+        assert k_cache.shape[1:] == (num_kv_heads, bs, dim) and v_cache.shape[1:] == (num_kv_heads, bs, vdim)
+        assert v_cache.shape[0] == k_cache.shape[0]
+    else:
+        bs = 1
+    gv = num_kv_heads * vdim
+    if v_first is not None:
+        assert v_first.shape == (t, gv) and v_first.dtype == torch.float32 and v_first.is_contiguous()
+    q = torch.empty((t, num_heads, dim), dtype=x.dtype, device=x.device)
+    kept = torch.empty((t, gv), dtype=torch.float32, device=x.device) if keep_v else None
+    _check(_LIB.vdamd_conv_norm_cache(
+        x.data_ptr(), x.stride(0), conv_weight.data_ptr(), state.data_ptr(), _i32(slots, "slots").data_ptr(),
+        _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(),
+        _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
+        _f32_vec(q_norm, dim, "q_norm").data_ptr(), _f32_vec(k_norm, dim, "k_norm").data_ptr(),
+        _ptr(v_first), _ptr(_f32_vec(v_lambda, 1, "v_lambda")) if v_first is not None else None, _ptr(kept),
+        q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _i32(slot_mapping, "slot_mapping").data_ptr(),
+        t, b, num_heads, num_kv_heads, dim, vdim, taps, bs, float(eps), 1 if has_prefill else 0, _dt(x), _stream()),
+        "conv_norm_cache")
+    return q, kept
+
+
+def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
+                          scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
+                          gate, max_query_len: int = 0):
+    t, h, d = q.shape
+    g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    assert q.is_contiguous() and q.dtype == k_cache.dtype == v_cache.dtype and h % g == 0
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[3] == d
+    assert v_cache.shape[:3] == k_cache.shape[:3] and dv <= UNIT_MAX_WIDTH
+    assert block_table.dim() == 2 and block_table.stride(1) == 1 and block_table.dtype == torch.int32
+    assert positions.shape[0] >= t and (token_seq is None or token_seq.shape[0] >= t)
+    assert token_seq is not None or t <= block_table.shape[0], "rows without a sequence"
+    gate_stride = 0
+    if gate is not None:
+        assert gate.shape == (t, h) and gate.stride(1) == 1 and gate.dtype == q.dtype
+        gate_stride = gate.stride(0)
+    out = torch.empty((t, h, dv), dtype=q.dtype, device=q.device)
+    _check(_LIB.vdamd_window_bias_attention(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
+        _ptr(_f32_vec(bias_scale, h, "bias_scale")), _ptr(_f32_vec(bias_rate, h, "bias_rate")),
+        _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, h, g, d, dv, bs,
+        int(window), int(keep_first), float(scale), float(softcap), _dt(q), _stream()), "window_bias_attention")
     return out

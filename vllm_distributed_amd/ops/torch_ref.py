@@ -433,3 +433,150 @@ def mla_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
         out.copy_(res)
         return out
     return res
+
+
+# ------------------------------------------------ single-gain RMS norms, PolyNorm, short convolutions with state
+def scalar_rms_norm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``x / sqrt(mean(x^2) + eps) * gain`` with one gain for the whole row, in fp32 arithmetic."""
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * gain.float()
+    return y.to(out_dtype)
+
+
+def scalar_norm_residual(y: torch.Tensor, post_gain: torch.Tensor, residual: torch.Tensor,
+                         next_gain: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype):
+    """``residual += norm(y) * post_gain`` in place on the fp32 residual stream; with ``next_gain`` also returns
+    ``norm(residual) * next_gain`` (the input of the sublayer that follows) in ``out_dtype``."""
+    residual.add_(scalar_rms_norm(y, post_gain, eps, torch.float32))
+    if next_gain is None:
+        return None
+    return scalar_rms_norm(residual, next_gain, eps, out_dtype)
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """``c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3`` with element-wise powers and ``N(u) = u / sqrt(mean(u^2) + eps)``
+    over the last dimension; fp32 arithmetic, result in ``z``'s dtype."""
+    zf = z.float()
+    c = coef.float()
+    out = torch.full_like(zf, float(c[3]))
+    p = zf
+    for i in range(3):
+        out = out + c[i] * p * torch.rsqrt(p.pow(2).mean(-1, keepdim=True) + eps)
+        p = p * zf
+    return out.to(z.dtype)
+
+
+def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
+               query_start_loc: torch.Tensor, seq_lens: torch.Tensor) -> torch.Tensor:
+    """Causal per-channel convolution over time of the packed rows ``x[T, C]`` with ``weight[C, taps]``:
+    ``y_t = sum_j weight[:, j] * u_(t - taps + 1 + j)``, zero before a sequence's first position.  Sequence ``i``
+    owns rows ``query_start_loc[i]:query_start_loc[i+1]``, the last positions of its ``seq_lens[i]`` tokens; the
+    ``taps - 1`` inputs in front of them come from ``state[slots[i]]`` (``[slots, taps - 1, C]``, oldest first),
+    which is left holding the last ``taps - 1`` inputs of the sequence.  Returns fp32 ``[T, C]``."""
+    taps = weight.shape[1]
+    r = taps - 1
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    wf = weight.float()
+    qsl, sls, sl = query_start_loc.tolist(), seq_lens.tolist(), slots.tolist()
+    for i, n_ctx in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        n = e - s
+        if n == 0:
+            continue
+        start = n_ctx - n
+        hist = state[sl[i]].float() if r else x.new_zeros((0, x.shape[1]), dtype=torch.float32)
+        if start < r:                      # positions before the sequence's start read as zero, whatever the slot held
+            hist = hist.clone()
+            hist[:r - start] = 0
+        u = torch.cat([hist, x[s:e].float()], 0)
+        acc = torch.zeros((n, x.shape[1]), dtype=torch.float32, device=x.device)
+        for j in range(taps):
+            acc += wf[:, j] * u[j:j + n]
+        y[s:e] = acc
+        if r:
+            state[sl[i]] = u[u.shape[0] - r:].to(state.dtype)
+    return y
+
+
+def conv_norm_cache(x: torch.Tensor, conv_weight: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
+                    query_start_loc: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, num_kv_heads: int,
+                    dim: int, vdim: int, q_norm: torch.Tensor, k_norm: torch.Tensor, eps: float,
+                    v_first: Optional[torch.Tensor], v_lambda: Optional[torch.Tensor], keep_v: bool,
+                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: torch.Tensor):
+    """Everything between the fused projection and the attention of a layer whose q / k / v pass through a short
+    convolution: ``x[T, C_x]`` holds ``[q | k | v | ...]`` (columns past the three are not touched);
+    ``short_conv`` over the first ``C`` columns, RMS norm of each q and k head with the ``[dim]`` weights,
+    ``v <- (1 - v_lambda) v + v_lambda v_first`` when ``v_first[T, Hkv * vdim]`` (fp32) is given, k and the mixed
+    v into the row caches ``[blocks, Hkv, block, dim | vdim]`` at ``slot_mapping``.  Returns ``(q[T, Hq, dim]``
+    in ``x``'s dtype, the unmixed fp32 ``v`` if ``keep_v`` else None``)``."""
+    t = x.shape[0]
+    qs, ks, vs = num_heads * dim, num_kv_heads * dim, num_kv_heads * vdim
+    c = qs + ks + vs
+    y = short_conv(x[:, :c], conv_weight, state, slots, query_start_loc, seq_lens)
+
+    def head_norm(u, w):
+        return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    q = head_norm(y[:, :qs].reshape(t, num_heads, dim), q_norm).to(x.dtype)
+    k = head_norm(y[:, qs:qs + ks].reshape(t, num_kv_heads, dim), k_norm)
+    v = y[:, qs + ks:].reshape(t, num_kv_heads, vdim)
+    kept = v.reshape(t, vs).clone() if keep_v else None
+    if v_first is not None:
+        lam = v_lambda.float()
+        v = (1.0 - lam) * v + lam * v_first.reshape(t, num_kv_heads, vdim)
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        valid = slot_mapping[:t] >= 0
+        sm = slot_mapping[:t][valid].long()
+        blk, off = sm // bs, sm % bs
+        k_cache[blk, :, off, :] = k[valid].to(k_cache.dtype)
+        v_cache[blk, :, off, :] = v[valid].to(v_cache.dtype)
+    return q, kept
+
+
+def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                          query_start_loc: torch.Tensor, seq_lens: torch.Tensor, scale: float, softcap: float,
+                          window: int, keep_first: int, bias_scale: Optional[torch.Tensor],
+                          bias_rate: Optional[torch.Tensor], sinks: Optional[torch.Tensor],
+                          gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """Causal attention over row caches ``k_cache[blocks, Hkv, block, D]`` / ``v_cache[blocks, Hkv, block, Dv]``.
+    A query at position ``i`` sees key ``j <= i`` when ``i - j < window`` (``window`` 0: no limit) or
+    ``j < keep_first``.  ``score = q.k * scale``, squashed to ``softcap * tanh(score / softcap)`` when
+    ``softcap > 0``, minus ``bias_scale[h] * ln(1 + bias_rate[h] * (i - j))``; ``sinks[h]`` adds ``exp(sinks[h])``
+    to the softmax denominator; ``gate[T, Hq]`` multiplies head ``h``'s output by ``sigmoid(gate[t, h])``.
+    fp32 arithmetic; returns ``[T, Hq, Dv]`` in ``q``'s dtype."""
+    t, hq, d = q.shape
+    hkv, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    g = hq // hkv
+    out = torch.zeros((t, hq, dv), dtype=torch.float32, device=q.device)
+    qsl, sls = query_start_loc.tolist(), seq_lens.tolist()
+    for i, sl in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        ql = e - s
+        if ql == 0:
+            continue
+        blocks = block_table[i, :(sl + bs - 1) // bs].long()
+        k = k_cache[blocks].permute(1, 0, 2, 3).reshape(hkv, -1, d)[:, :sl].float().repeat_interleave(g, dim=0)
+        v = v_cache[blocks].permute(1, 0, 2, 3).reshape(hkv, -1, dv)[:, :sl].float().repeat_interleave(g, dim=0)
+        qi = q[s:e].float().transpose(0, 1)
+        sc = torch.matmul(qi, k.transpose(1, 2)) * scale
+        if softcap > 0:
+            sc = torch.tanh(sc / softcap) * softcap
+        qpos = torch.arange(sl - ql, sl, device=q.device).unsqueeze(1)
+        kpos = torch.arange(sl, device=q.device).unsqueeze(0)
+        dist = (qpos - kpos).clamp(min=0).float()
+        if bias_scale is not None:
+            sc = sc - bias_scale.float().view(-1, 1, 1) * torch.log1p(bias_rate.float().view(-1, 1, 1) * dist)
+        seen = kpos <= qpos
+        if window > 0:
+            seen = seen & (((qpos - kpos) < window) | (kpos < keep_first))
+        sc = sc.masked_fill(~seen, float("-inf"))
+        if sinks is not None:
+            col = sinks.float().view(-1, 1, 1).expand(hq, ql, 1)
+            p = torch.softmax(torch.cat([sc, col], dim=-1), -1)[..., :-1]
+        else:
+            p = torch.softmax(sc, -1)
+        out[s:e] = torch.matmul(p, v).transpose(0, 1)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
+    return out.to(q.dtype)

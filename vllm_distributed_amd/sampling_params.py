@@ -41,6 +41,9 @@ class SamplingParams:
     # "last" | "mean": return the pooled final hidden state of the prompt (embeddings, scoring)
     # with the request's single output token; the request then ends after that token
     pooling: Optional[str] = None
+    # every token of the request is given by the caller (a token trace replayed step by step): nothing is sampled,
+    # the request runs until the caller ends it
+    score_only: bool = False
     guided_regex: Optional[str] = None                   # the output matches this regular expression
     guided_json: Optional[Any] = None                    # the output is JSON satisfying this schema (dict or str)
     guided_grammar: Optional[str] = None                 # the output is a sentence of this EBNF grammar (start rule: root)

@@ -46,6 +46,7 @@ class InputBatch:
         self.has_penalty = np.zeros(n, dtype=bool)
         self.num_prompt_logprobs = np.full(n, -1, dtype=np.int32)
         self.pooling = np.zeros(n, dtype=np.int8)           # 0 none, 1 last token, 2 mean over the prompt
+        self.score_only = np.zeros(n, dtype=bool)             # every token is given: the row is never sampled
         self.has_adjust = np.zeros(n, dtype=bool)             # logit bias / allow / ban lists / min_tokens
         self.lora_id = np.zeros(n, dtype=np.int32)              # 0 = base model
         self.req_ids: List[Optional[str]] = [None] * n
@@ -91,6 +92,7 @@ class InputBatch:
         self.repetition[row] = sp.repetition_penalty
         self.has_penalty[row] = sp.has_penalties
         self.has_adjust[row] = sp.has_logit_adjust
+        self.score_only[row] = bool(getattr(sp, "score_only", False))
         self.num_prompt_logprobs[row] = -1 if sp.prompt_logprobs is None else sp.prompt_logprobs
         self.pooling[row] = {None: 0, "last": 1, "mean": 2}[sp.pooling]
         self.grammar[row] = None
@@ -136,6 +138,7 @@ class InputBatch:
         self.num_blocks[row] = 0
         self.lora_id[row] = 0
         self.has_adjust[row] = False
+        self.score_only[row] = False
         self.num_prompt_logprobs[row] = -1
         self.pooling[row] = 0
         self.grammar[row] = None

@@ -82,7 +82,7 @@ class PendingSample:
     lazy_step_result = True       # executors call .get() / .wait() on results carrying this mark
     __slots__ = ("runner", "step_id", "req_ids", "nreq", "sel", "rows", "gens", "pos", "tokens",
                  "event", "logprobs", "timing", "marks", "_result", "prompt_logprobs", "_lock", "_toks",
-                 "_published", "kv_sent", "kv_recv", "pooled", "counts", "drafts", "_accepted", "proposals")
+                 "_published", "kv_sent", "kv_recv", "pooled", "counts", "drafts", "_accepted", "proposals", "logits")
 
     def __init__(self, runner: "ModelRunner", step_id: int, req_ids: List[str], sel: Optional[np.ndarray],
                  rows: Optional[np.ndarray], pos: Optional[np.ndarray], tokens: Optional[torch.Tensor],
@@ -94,6 +94,7 @@ class PendingSample:
         self.logprobs, self.timing, self.marks = logprobs, timing, marks
         self.prompt_logprobs = None
         self.pooled = None                   # (req ids, [k, H] float32 device tensor)
+        self.logits = None                   # (req ids, rows per request, [sum, vocab] float32 host tensor)
         # speculative decoding: sampled positions per selected request, and each one's draft tokens (or None)
         self.counts: Optional[np.ndarray] = None
         self.drafts: Optional[List[Optional[List[int]]]] = None
@@ -151,6 +152,13 @@ class PendingSample:
             if self.pooled is not None:
                 ids, vecs = self.pooled
                 pooled = dict(zip(ids, vecs.cpu().tolist()))
+            logits = None
+            if self.logits is not None:
+                ids, counts, vals = self.logits
+                vals, logits, off = vals.numpy(), {}, 0
+                for rid, c in zip(ids, counts):
+                    logits[rid] = vals[off:off + c]
+                    off += c
             timing = self.timing
             if timing is not None and self.marks is not None:
                 timing.update(self.marks.resolve())
@@ -159,7 +167,7 @@ class PendingSample:
                                              prompt_logprobs=self.prompt_logprobs, pooled=pooled,
                                              finished_sending=self.kv_sent or None,
                                              finished_recving=self.kv_recv or None,
-                                             draft_token_ids=self.proposals)
+                                             draft_token_ids=self.proposals, logits=logits)
             return self._result
 
     def publish(self) -> None:
@@ -240,6 +248,7 @@ class ModelRunner:
         self.batch = InputBatch(self.max_num_reqs, self.max_model_len, self.block_size,
                                 self.model_config.vocab_size, self.model_config.seed)
         self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
+        self.state_tensors: List[torch.Tensor] = []
         self.graphs: Dict[int, DecodeGraph] = {}
         # batch size -> [(context limit, graph)] ascending; the last entry is also graphs[batch size]
         self.graph_ctx: Dict[int, List[Tuple[int, DecodeGraph]]] = {}
@@ -247,6 +256,7 @@ class ModelRunner:
         self.graph_pool = None
         self.graph_fallback_reason: Optional[str] = "not captured yet"
         self._static: Dict[str, torch.Tensor] = {}
+        self._stage_copied = None         # event behind the last step's copies out of the pinned staging tensors
         self.decode_workspace: Optional[torch.Tensor] = None
         self.draft = None                 # worker.draft_model.DraftProposer (draft-model speculation)
         # vision-language requests: their images (multimodal.MultiModalInput) and the projected features of
@@ -286,12 +296,15 @@ class ModelRunner:
         mode = envs.VDAMD_TP_OVERLAP
         if (self.is_gpu and self.pp.world_size == 1 and hasattr(self.model, "forward_overlapped")
                 and getattr(self.model, "tp_fusions", True) and (mode == "force" or (mode == "auto" and self.tp.world_size > 1))):
-            self.comm_stream = torch.cuda.Stream(priority=-1)
+            self.comm_stream = torch.cuda.Stream()
         self.pp_link = None
         if self.pp.world_size > 1:
             from ..parallel.pipeline import PipelineLink
             self.pp_link = PipelineLink(self.pp, self.device, use_rccl=envs.VDAMD_COMM_BACKEND in ("auto", "rccl"))
         sc = self.vllm_config.speculative_config
+        if sc is not None and getattr(self.model, "has_request_state", False):
+            raise ValueError("speculative decoding is not supported for a model with per-request layer state: "
+                             "a rejected draft would have advanced it")
         if sc is not None and sc.worker_side:
             from .draft_model import DraftProposer, HiddenStateProposer, MedusaProposer
             if sc.reads_target_hidden:
@@ -321,11 +334,23 @@ class ModelRunner:
             # one shared latent row per token, held in two layouts: (rank + rope) + rank values, which the
             # spec's "2 x heads x head_dim" states as one head of half that sum
             heads, width = 1, a.kv_values_per_token() // 2
+        # layers of unlike shape (each with its own heads and key / value sizes): the sum over the layers is stated
+        per_token = sum(l.kv_values_per_token() for l in layers)
+        uniform = per_token == 2 * len(layers) * heads * width
+        state = sum(l.state_values_per_slot() for l in self._state_layers()) * self.model_config.dtype_bytes
         return KVCacheSpec(num_layers=len(layers), num_kv_heads=heads, head_dim=width,
                            block_size=self.block_size, dtype_bytes=dtype_bytes,
                            sliding_window=max(windows) if windows and min(windows) > 0 else None,
+                           keep_first=max(int(getattr(l, "keep_first", 0) or 0) for l in layers),
+                           values_per_token=None if uniform else per_token,
+                           state_bytes_per_request=state,
                            extra_bytes_per_block=(self.draft.kv_bytes_per_block(self.block_size, dtype_bytes)
                                                   if self.draft is not None else 0))
+
+    def _state_layers(self) -> list:
+        """Layers that keep per-request state besides the KV cache (short convolutions, recurrences)."""
+        fn = getattr(self.model, "state_layers", None)
+        return list(fn()) if fn is not None else []
 
     @torch.inference_mode()
     def profile_run(self) -> None:
@@ -366,6 +391,13 @@ class ModelRunner:
                 scales = tuple(t.to(self.device) for t in scales)
             attn.bind_kv_cache(k, v, scales)
             self.kv_caches.append((k, v))
+        # per-request state: one slot per row of the persistent batch, never cleared (a layer reads nothing of a
+        # slot that lies before its sequence's start)
+        self.state_tensors = []
+        for layer in self._state_layers():
+            st = torch.zeros(layer.state_shape(self.max_num_reqs), dtype=self.model_config.torch_dtype, device=self.device)
+            layer.bind_state(st)
+            self.state_tensors.append(st)
         if self.draft is not None:
             self.draft.allocate_kv(num_blocks, self.block_size, dtype, fp8)
         logger.info("KV cache: %d blocks x %d tokens (%.2f GiB)", num_blocks, self.block_size,
@@ -402,6 +434,11 @@ class ModelRunner:
             if toks and not samples_here:
                 # stages that do not sample learn new tokens from the scheduler
                 b.append_tokens(row, toks)
+        for rid, toks in (so.appended_prompt_tokens or {}).items():
+            row = b.row_of.get(rid)          # the front end lengthened a known request's prompt (token replay)
+            if row is not None:
+                b.append_tokens(row, toks)
+                b.num_prompt_tokens[row] += len(toks)
         if so.scheduled_spec_decode_tokens:
             # draft tokens sit behind the last real token as this step's extra inputs; they are not
             # part of the request (num_tokens stays) until the step has verified them
@@ -490,7 +527,7 @@ class ModelRunner:
         slot_mapping = (blk * self.block_size + positions % self.block_size).astype(np.int32)
         max_blocks = int(cdiv(int(seq_lens.max()), self.block_size))
         # which requests reach the end of their known tokens -> sample
-        sample_mask = seq_lens >= b.num_tokens[rows]
+        sample_mask = (seq_lens >= b.num_tokens[rows]) & ~b.score_only[rows]
         spec = so.scheduled_spec_decode_tokens
         return dict(spec=spec if spec else None,
                     req_ids=req_ids, rows=rows, n_sched=n_sched, num_decodes=num_decodes,
@@ -522,6 +559,8 @@ class ModelRunner:
             max_query_len=int(n_sched.max()), max_seq_len=int(p["seq_lens"].max()),
             max_decode_seq_len=int(p["seq_lens"][:nd].max()) if nd else 0,
             decode_workspace=self.decode_workspace)
+        if self.state_tensors:
+            md.state_slots = self._to_dev(p["rows"])
         if nreq > nd:
             pq = p["qsl"][nd:] - p["qsl"][nd]
             md.prefill_query_start_loc = self._to_dev(pq)
@@ -628,6 +667,7 @@ class ModelRunner:
         pooled = None
         if nd < nreq and self.batch.pooling[p["rows"][nd:]].any():
             pooled = self._pool(hidden, p)
+        wanted_logits = self._logits_at(hidden, p, so.logits_wanted) if so.logits_wanted else None
         sample_mask = p["sample_mask"]
         sel = rows_sel = pos_sel = host_tokens = event = logprobs_sel = None
         counts = drafts_sel = None
@@ -683,7 +723,7 @@ class ModelRunner:
             self._last_end_mark = marks.end
             if self.is_gpu:
                 event = marks.end
-        elif self.is_gpu and sel is not None:
+        elif self.is_gpu and (sel is not None or wanted_logits is not None):
             event = torch.cuda.Event()
             event.record()
         # host time of this call: building inputs, and launching (not running) the device work
@@ -696,6 +736,7 @@ class ModelRunner:
         pending.counts, pending.drafts = counts, drafts_sel
         pending.proposals = proposals
         pending.pooled = pooled
+        pending.logits = wanted_logits
         pending.kv_sent, pending.kv_recv = kv_sent, kv_recv
         self._pending.append(pending)
         report_all = self.kv_connector is not None      # the executor aggregates transfer reports of all ranks
@@ -777,7 +818,8 @@ class ModelRunner:
             num_decodes=n, num_decode_tokens=n, num_prefills=0, num_prefill_tokens=0,
             slot_mapping=md.slot_mapping[s:e], block_table=md.block_table[s:e], seq_lens=md.seq_lens[s:e],
             query_start_loc=md.query_start_loc[:n + 1], max_query_len=1, max_seq_len=md.max_seq_len,
-            max_decode_seq_len=md.max_decode_seq_len, decode_workspace=md.decode_workspace)
+            max_decode_seq_len=md.max_decode_seq_len, decode_workspace=md.decode_workspace,
+            state_slots=None if md.state_slots is None else md.state_slots[s:e])
 
     def _forward_decode(self, md: AttentionMetadata, input_ids: torch.Tensor, positions: torch.Tensor):
         """Pure-decode forward on a single pipeline stage, overlapped when enabled.  Leaves the TP
@@ -821,7 +863,7 @@ class ModelRunner:
         """``(hidden, residual)`` of the previous stage for ``total`` tokens: one message, received
         on the pipeline link's own stream.  ``static``: into the buffers a captured graph reads."""
         h = self.model_config.hidden_size
-        dtype = self.model_config.torch_dtype
+        dtype = getattr(self.model, "residual_dtype", None) or self.model_config.torch_dtype
         want_res = self._pp_sends_residual()
         if static:
             hidden = self._static["pp_hidden"][:total]
@@ -885,6 +927,32 @@ class ModelRunner:
                     d.setdefault(t_id, t_lp)
                 logprobs.append([d])
         return tokens.to(torch.int32), logprobs
+
+    def _logits_at(self, hidden: torch.Tensor, p: dict, wanted: Dict[str, List[int]]):
+        """Full-vocabulary logits at the places a step's caller asked for: ``wanted[req] = indices among the
+        tokens the request runs in this step``.  Returns ``(req ids, rows per request, [sum, vocab] fp32 on the
+        host, copied without blocking)`` in the order of ``wanted``."""
+        where = {rid: i for i, rid in enumerate(p["req_ids"])}
+        ids, counts, idx = [], [], []
+        for rid, places in wanted.items():
+            i = where.get(rid)
+            if i is None or not places:
+                continue
+            n = int(p["n_sched"][i])
+            if min(places) < 0 or max(places) >= n:
+                raise ValueError(f"logits of {rid} asked at {places}, but the step runs {n} of its tokens")
+            ids.append(rid)
+            counts.append(len(places))
+            idx.extend(int(p["qsl"][i]) + int(k) for k in places)
+        if not ids:
+            return None
+        rows = hidden.index_select(0, self._to_dev(np.asarray(idx, dtype=np.int64), torch.int64))
+        vals = self.model.compute_logits(rows).float()
+        if self.is_gpu:
+            host = torch.empty(vals.shape, dtype=torch.float32, pin_memory=True)
+            host.copy_(vals, non_blocking=True)
+            vals = host
+        return ids, counts, vals
 
     def _pool(self, hidden: torch.Tensor, p: dict):
         """Pooled final hidden states of the prefill rows that asked for them (embedding / scoring
@@ -1117,6 +1185,7 @@ class ModelRunner:
             "seq_lens": torch.zeros(max_bs, dtype=torch.int32, device=dev),
             "block_table": torch.zeros(max_bs, mb, dtype=torch.int32, device=dev),
             "qsl": torch.arange(max_bs + 1, dtype=torch.int32, device=dev),
+            "state_slots": torch.zeros(max_bs, dtype=torch.int32, device=dev),
         }
         if self.is_gpu:
             # pinned staging so one H2D per tensor per step
@@ -1130,7 +1199,8 @@ class ModelRunner:
             slot_mapping=s["slot_mapping"][:bs], block_table=s["block_table"][:bs],
             seq_lens=s["seq_lens"][:bs], query_start_loc=s["qsl"][:bs + 1],
             max_query_len=1, max_seq_len=max_seq_len, max_decode_seq_len=max_seq_len,
-            decode_workspace=self.decode_workspace)
+            decode_workspace=self.decode_workspace,
+            state_slots=s["state_slots"][:bs] if self.state_tensors else None)
 
     @torch.inference_mode()
     def capture_graphs(self) -> None:
@@ -1143,7 +1213,9 @@ class ModelRunner:
             return
         first = self.model.attention_layers()[0]
         kernel_head_dim = first.head_dim      # (padded to a kernel size where needed)
-        if getattr(first, "latent", False):
+        if getattr(first, "row_cache", False):        # attention over plain row caches: its kernels take any head size
+            kernel_ok = ops.hip_available()
+        elif getattr(first, "latent", False):
             kernel_ok = ops.mla_kernel_ok(first.head_dim, first.v_dim, self.model_config.torch_dtype)
         else:
             kernel_ok = ops.hip_supports_head_dim(kernel_head_dim)
@@ -1264,10 +1336,19 @@ class ModelRunner:
         s, st = self._static, self._stage
         n, bs = len(p["req_ids"]), g.batch_size
         mb = p["max_blocks"]
+        # the pinned staging tensors are read by the device when the copies below run, not when they are issued:
+        # a step that nobody waits for (nothing sampled, no logits asked) must not have them rewritten under it
+        if self._stage_copied is not None:
+            self._stage_copied.synchronize()
         st["input_ids"][:n] = torch.from_numpy(p["input_ids"])
         st["positions"][:n] = torch.from_numpy(p["positions"])
         st["slot_mapping"][:n] = torch.from_numpy(p["slot_mapping"])
         st["seq_lens"][:n] = torch.from_numpy(p["seq_lens"])
+        if self.state_tensors:
+            st["state_slots"][:n] = torch.from_numpy(p["rows"].astype(np.int32))
+            if n < bs:       # padding rows run the layers too: their state goes to a row no request holds
+                st["state_slots"][n:bs] = self._spare_state_rows(p["rows"], bs - n)
+            s["state_slots"][:bs].copy_(st["state_slots"][:bs], non_blocking=True)
         st["block_table"][:n, :mb] = torch.from_numpy(self.batch.block_table[p["rows"], :mb])
         if n < bs:      # padding rows: no cache write, zero-length attention
             st["slot_mapping"][n:bs] = -1
@@ -1278,6 +1359,9 @@ class ModelRunner:
             s[k][:bs].copy_(st[k][:bs], non_blocking=True)
         s["block_table"][:n, :mb].copy_(st["block_table"][:n, :mb], non_blocking=True)
         self._patch_unknown_inputs(s["input_ids"], p)
+        if self._stage_copied is None:
+            self._stage_copied = torch.cuda.Event()
+        self._stage_copied.record()
         if self.pp_link is not None:
             # the stage's layers are the graph; the transfers around it run on the link's streams
             if not self.pp.is_first_rank:
@@ -1292,6 +1376,14 @@ class ModelRunner:
         if g.aux is not None:
             self.model.last_aux = g.aux
         return g.output
+
+    def _spare_state_rows(self, used: np.ndarray, k: int) -> torch.Tensor:
+        """``k`` state slots for the padding rows of a captured batch: rows of the persistent batch that no request
+        holds (a padded batch is smaller than ``max_num_seqs``, so there are enough), else row 0's neighbours."""
+        free = np.setdiff1d(np.arange(self.max_num_reqs), np.asarray(list(self.batch.row_of.values()), dtype=np.int64))
+        if len(free) == 0:
+            raise RuntimeError("no free state slot for the padding rows of a decode graph")
+        return torch.from_numpy(np.resize(free, k).astype(np.int32))
 
     # ----------------------------------------------------------------- warmup
     @torch.inference_mode()
