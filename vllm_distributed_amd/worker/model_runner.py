@@ -392,10 +392,11 @@ class ModelRunner:
             attn.bind_kv_cache(k, v, scales)
             self.kv_caches.append((k, v))
         # per-request state: one slot per row of the persistent batch, never cleared (a layer reads nothing of a
-        # slot that lies before its sequence's start)
+        # slot that lies before its sequence's start), and one spare slot behind them for the padding rows of
+        # captured decode batches
         self.state_tensors = []
         for layer in self._state_layers():
-            st = torch.zeros(layer.state_shape(self.max_num_reqs), dtype=self.model_config.torch_dtype, device=self.device)
+            st = torch.zeros(layer.state_shape(self.max_num_reqs + 1), dtype=self.model_config.torch_dtype, device=self.device)
             layer.bind_state(st)
             self.state_tensors.append(st)
         if self.draft is not None:
@@ -1185,7 +1186,7 @@ class ModelRunner:
             "seq_lens": torch.zeros(max_bs, dtype=torch.int32, device=dev),
             "block_table": torch.zeros(max_bs, mb, dtype=torch.int32, device=dev),
             "qsl": torch.arange(max_bs + 1, dtype=torch.int32, device=dev),
-            "state_slots": torch.zeros(max_bs, dtype=torch.int32, device=dev),
+            "state_slots": torch.full((max_bs,), self.max_num_reqs, dtype=torch.int32, device=dev),
         }
         if self.is_gpu:
             # pinned staging so one H2D per tensor per step
@@ -1346,8 +1347,8 @@ class ModelRunner:
         st["seq_lens"][:n] = torch.from_numpy(p["seq_lens"])
         if self.state_tensors:
             st["state_slots"][:n] = torch.from_numpy(p["rows"].astype(np.int32))
-            if n < bs:       # padding rows run the layers too: their state goes to a row no request holds
-                st["state_slots"][n:bs] = self._spare_state_rows(p["rows"], bs - n)
+            if n < bs:       # padding rows run the layers too: their state goes to the spare slot no request holds
+                st["state_slots"][n:bs] = self.max_num_reqs
             s["state_slots"][:bs].copy_(st["state_slots"][:bs], non_blocking=True)
         st["block_table"][:n, :mb] = torch.from_numpy(self.batch.block_table[p["rows"], :mb])
         if n < bs:      # padding rows: no cache write, zero-length attention
@@ -1376,14 +1377,6 @@ class ModelRunner:
         if g.aux is not None:
             self.model.last_aux = g.aux
         return g.output
-
-    def _spare_state_rows(self, used: np.ndarray, k: int) -> torch.Tensor:
-        """``k`` state slots for the padding rows of a captured batch: rows of the persistent batch that no request
-        holds (a padded batch is smaller than ``max_num_seqs``, so there are enough), else row 0's neighbours."""
-        free = np.setdiff1d(np.arange(self.max_num_reqs), np.asarray(list(self.batch.row_of.values()), dtype=np.int64))
-        if len(free) == 0:
-            raise RuntimeError("no free state slot for the padding rows of a decode graph")
-        return torch.from_numpy(np.resize(free, k).astype(np.int32))
 
     # ----------------------------------------------------------------- warmup
     @torch.inference_mode()
