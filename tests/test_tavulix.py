@@ -44,7 +44,7 @@ CONFIGS = {
                           layer(mixer(3, 3, 8, 8, 2, 400, 0, v_mix=False), 32),
                           layer(mixer(2, 2, 16, 16, 3, 6, 6, v_mix=False))], width=32, vocab=50),
     # a window that spans pages of 16 tokens and a kept prefix longer than a page
-    "paged": config([layer(mixer(4, 1, 32, 16, 3, 37, 19), 96), layer(mixer(4, 4, 16, 16, 3, 70, 1), 96)], width=64),
+    "paged": config([layer(mixer(4, 1, 32, 16, 3, 37, 19), 96), layer(mixer(4, 1, 16, 16, 3, 70, 1), 96)], width=64),
 }
 
 
