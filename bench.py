@@ -139,6 +139,11 @@ def _parse():
     ap.add_argument("--alt-parallelism", type=str, default="pp",
                     help="second layout measured in a child process after the headline when N > 1 ('none' = skip)")
     ap.add_argument("--alt-timeout", type=float, default=900.0)
+    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix"],
+                    help="instead of the headline: prefill and decode throughput of this model family at a few layer "
+                         "sizes beside the closest existing family (Gemma-2) at equal size, random weights, one GPU")
+    ap.add_argument("--compare-sizes", type=str, default="small,medium",
+                    help="with --family-compare: which of small / medium / large to run")
     ap.add_argument("--device", type=str, default="cuda", choices=["cuda", "cpu"],
                     help="cpu = gloo rehearsal of the multi-rank path with a tiny model (not a measurement)")
     return ap.parse_args()
@@ -192,8 +197,82 @@ def _measure_alt_layout(args, n: int) -> dict:
         return {"parallelism": f"tp{tp}xpp{pp}", "error": repr(e)[-600:]}
 
 
+COMPARE_SIZES = {
+    "tiny": dict(width=128, heads=4, kv=2, dim=64, ff=256, layers=2, window=32, prompt=96, prompts=2, batch=4),
+    # width, heads, kv heads, head size, feed-forward, layers, window, prompt length, prefill prompts, decode batch
+    "small": dict(width=1024, heads=8, kv=2, dim=128, ff=4096, layers=4, window=512, prompt=1024, prompts=16, batch=64),
+    "medium": dict(width=2048, heads=16, kv=4, dim=128, ff=8192, layers=4, window=1024, prompt=2048, prompts=8, batch=128),
+    "large": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, layers=2, window=4096, prompt=4096, prompts=4, batch=128),
+}
+
+
+def _compare_models(z: dict) -> dict:
+    """The same layer sizes as a Tavulix config and as a Gemma-2 config (norms on both sides of every sublayer,
+    capped scores, a window, capped logits: the closest family the framework has)."""
+    vocab, positions = 32000, 8192
+    mixer = {"conv": 4, "dim": z["dim"], "vdim": z["dim"], "heads": z["heads"], "kv_heads": z["kv"],
+             "scale": z["dim"] ** -0.5, "softcap": 30.0, "v_mix": True, "mask": {"size": z["window"], "keep_first": 8}}
+    tav = {"architecture": "Tavulix", "vocab": vocab, "width": z["width"], "max_positions": positions,
+           "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+           "layers": [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": z["ff"]}}] * z["layers"]}
+    gem = {"hidden_size": z["width"], "num_attention_heads": z["heads"], "num_key_value_heads": z["kv"],
+           "head_dim": z["dim"], "intermediate_size": z["ff"], "num_hidden_layers": z["layers"],
+           "sliding_window": z["window"], "layer_types": ["sliding_attention"] * z["layers"],
+           "query_pre_attn_scalar": z["dim"], "vocab_size": vocab, "max_position_embeddings": positions,
+           "torch_dtype": "bfloat16"}
+    return {"tavulix": ("tavulix-tiny", tav), "gemma2": ("gemma2-tiny", gem)}
+
+
+def run_family_compare(args) -> None:
+    """Prefill throughput (``prompts`` prompts of ``prompt`` tokens, one generated token each) and decode
+    throughput (``batch`` sequences, 64 further tokens each; the prefill time measured the same way is taken off)
+    through ``LLM.generate``, per family and size; one JSON line."""
+    import numpy as np
+    import torch
+    from vllm_distributed_amd import LLM, SamplingParams
+    os.environ.setdefault("VLLM_LOGGING_LEVEL", "WARNING")
+    rows = []
+    for size in [s for s in args.compare_sizes.split(",") if s]:
+        z = COMPARE_SIZES[size]
+        for family, (base, over) in _compare_models(z).items():
+            llm = LLM(model=base, hf_overrides=over, dtype=args.dtype, device=args.device, load_format="dummy",
+                      max_model_len=z["prompt"] + 128, max_num_seqs=max(z["batch"], z["prompts"]),
+                      max_num_batched_tokens=8192, gpu_memory_utilization=0.5, enforce_eager=args.enforce_eager,
+                      enable_prefix_caching=False)
+            rng = np.random.default_rng(0)
+            vocab = 32000
+
+            def timed(n_prompts, prompt_len, new_tokens):
+                prompts = [rng.integers(0, 32000, prompt_len).tolist() for _ in range(n_prompts)]
+                if args.device == "cuda":
+                    torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=new_tokens, ignore_eos=True))
+                if args.device == "cuda":
+                    torch.cuda.synchronize()
+                return time.perf_counter() - t0
+            try:
+                timed(2, 64, 4)                                         # warm-up
+                timed(z["prompts"], z["prompt"], 1)
+                t_pre = min(timed(z["prompts"], z["prompt"], 1) for _ in range(2))
+                ctx = min(z["prompt"], 1024)
+                t_a = min(timed(z["batch"], ctx, 1) for _ in range(2))
+                t_b = min(timed(z["batch"], ctx, 65) for _ in range(2))
+                rows.append({"family": family, "size": size,
+                             "prefill_tokens_per_s": round(z["prompts"] * z["prompt"] / t_pre, 1),
+                             "decode_tokens_per_s": round(z["batch"] * 64 / max(t_b - t_a, 1e-9), 1),
+                             "decode_ms_per_step": round(1e3 * (t_b - t_a) / 64, 3), "shape": z})
+            finally:
+                llm.shutdown()
+    print(json.dumps({"metric": "family_compare", "family": args.family_compare, "dtype": args.dtype,
+                      "data": "synthetic", "rows": rows}), flush=True)
+
+
 def main() -> None:
     args = _parse()
+    if args.family_compare:
+        run_family_compare(args)
+        return
     n = args.gpus
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

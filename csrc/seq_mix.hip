@@ -8,9 +8,14 @@
 //                          from the chunk itself or from a per-request state slot), per-head RMS norm of q and k,
 //                          value mixing, k / v into row caches, q out
 //   conv_state_update      the last taps-1 projected rows of every sequence into its state slot
-//   window_bias_attention  attention over row caches [blocks, Hkv, block, D] / [.., Dv]: causal window that keeps
-//                          the first keys, score cap, logarithmic distance bias, sink in the denominator, sigmoid
-//                          gate on the output; one wave per (token, query head), online softmax in fp32
+//   window_bias_attention  attention over the caches K [blocks, Hkv, block, D] (key rows) and V [blocks, Hkv,
+//                          block / 8, Dv, 8] (8 keys side by side per channel: the V^T operand of the matrix cores
+//                          is one 16-byte load): causal window that keeps the first keys, score cap, logarithmic
+//                          distance bias, sink in the denominator, sigmoid gate on the output, online softmax in
+//                          fp32.  Two kernels: a matrix-core one for bf16 (16 query rows x 32 keys per wave and
+//                          step, softmax weights fed to the matrix cores as a high and a low bf16 part so that they
+//                          keep fp32 precision), and a plain one (any head size, fp16 / fp32) with one wave per
+//                          (token, query head)
 //
 // Element types: bf16 / fp16 / fp32 for activations and caches (fp32: the model runs entirely in 32-bit).
 #include "common.h"
@@ -191,11 +196,20 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
     }
     if (slot < 0 || a.k_cache == nullptr) continue;
     const long blk = slot / a.block_size, off = slot % a.block_size;
-    T* dst = (kind == 1 ? (T*)a.k_cache : (T*)a.v_cache) + ((blk * a.G + head) * a.block_size + off) * (long)width;
+    if (kind == 1) {
+      T* dst = (T*)a.k_cache + ((blk * a.G + head) * a.block_size + off) * (long)width;
 #pragma unroll
-    for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
-      const int cl = lane + it * 64;
-      if (cl < width) stf(dst + cl, acc[it]);
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) stf(dst + cl, acc[it]);
+      }
+    } else {                                      // [blocks, G, bs / 8, Dv, 8]
+      T* dst = (T*)a.v_cache + (((blk * a.G + head) * (a.block_size >> 3) + (off >> 3)) * (long)width) * 8 + (off & 7);
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) stf(dst + (long)cl * 8, acc[it]);
+      }
     }
   }
 }
@@ -311,7 +325,7 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
       sc = RowDot<T, VEC>::run(kc + row * a.D, sq, a.D) * a.scale;
       if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
       if (a.bias_scale) sc -= r1 * log1pf(r2 * (float)(pos - j));
-      vrow = row * a.Dv;
+      vrow = (((blk * a.G + g) * (a.block_size >> 3) + ((j % a.block_size) >> 3)) * (long)a.Dv) * 8 + (j & 7);
     }
     const float m_new = fmaxf(m, wave_max(sc));
     const float p = f < total ? expf(sc - m_new) : 0.f;
@@ -330,7 +344,7 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
 #pragma unroll
       for (int i = 0; i < ATTN_V_PER_LANE; ++i) {
         const int c = cl0 + i * cw;
-        if (c < a.Dv) acc[i] += pj * ldf(vr + c);
+        if (c < a.Dv) acc[i] += pj * ldf(vr + (long)c * 8);
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -363,6 +377,193 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
       const int c = cl0 + i * cw;
       if (c < a.Dv) stf(o + c, acc[i] * mul);
     }
+  }
+}
+
+
+// ------------------------------------------------------------------- attention on the matrix cores (bf16)
+// A wave owns 16 query rows = `tpw` consecutive tokens of one sequence x `hp` heads of one GQA group (row r: token
+// r / hp, head r % hp) and walks the visible keys 32 at a time.  Per step: S^T = K Q^T (two 16-key tiles whose rows
+// interleave so that a lane ends up with 8 consecutive keys of ITS query row), cap / bias / mask / online softmax in
+// fp32 per lane, O^T += V^T P^T with P split into bf16 high and low parts.  Everything a query row needs (max, sum,
+// rescale factor, its O^T column) lives in the lanes with l % 16 == row.  With `kw` > 1 the block's waves take the
+// key steps in turn for the same rows and are merged through LDS (decode: few rows, many keys).
+template <int DT, int VT>
+__global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArgs a, const int* __restrict__ qsl,
+                                                                         const int* __restrict__ seq_lens, int hp,
+                                                                         int tpw, int kw) {
+  using T = bf16_t;
+  using V8 = bf16x8;
+  extern __shared__ float lds[];
+  constexpr int D = 32 * DT, DV = 16 * VT;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int r16 = lane & 15, g4 = lane >> 4;
+  const int s = blockIdx.z;
+  const int qpg = a.H / a.G;
+  const int hchunks = (qpg + hp - 1) / hp;
+  const int g = blockIdx.y / hchunks, hc = blockIdx.y % hchunks;
+  const int tw = nwaves / kw;                     // waves over tokens
+  const int wt = wave / kw, wk = wave % kw;
+  const int q0 = qsl[s], n_tok = qsl[s + 1] - q0;
+  const int tok0 = (blockIdx.x * tw + wt) * tpw;  // first token (within the step's rows of the sequence) of this wave
+  if (tok0 >= n_tok && kw == 1) return;
+  const bool wave_live = tok0 < n_tok;
+  const int start = seq_lens[s] - n_tok;          // position of the sequence's first row in this step
+  // ---- this lane's query row
+  const int tl = r16 / hp, hh = r16 % hp;
+  const int tok = tok0 + tl;
+  const bool row_ok = wave_live && tl < tpw && tok < n_tok && hc * hp + hh < qpg;
+  const int h = g * qpg + min(hc * hp + hh, qpg - 1);
+  const long trow = q0 + min(tok, max(n_tok - 1, 0));
+  const int pos = start + min(tok, max(n_tok - 1, 0));
+  V8 qf[DT];
+  {
+    const T* qp = (const T*)a.q + (trow * a.H + h) * (long)D + 8 * g4;
+#pragma unroll
+    for (int k = 0; k < DT; ++k) {
+      if (row_ok) qf[k] = ld8<T>(qp + 32 * k);
+      else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[k][j] = (T)0.f;
+      }
+    }
+  }
+  const float r1 = a.bias_scale ? a.bias_scale[h] : 0.f;      // (r1 ln(x) on the log2 scale is r1 log2(x))
+  const float r2 = a.bias_rate ? a.bias_rate[h] : 0.f;
+  const float scale2 = a.scale * LOG2E;
+  // ---- key steps of the wave: [0, kept) and [window start of its first row, position of its last row]
+  const int p_first = start + min(tok0, max(n_tok - 1, 0));
+  const int p_last = start + min(tok0 + tpw - 1, max(n_tok - 1, 0));
+  const int lo_min = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  const int nkeep = a.window > 0 ? min(a.keep_first, lo_min) : 0;
+  int start_b = lo_min & ~31;
+  int n_a = (nkeep + 31) >> 5;
+  if (start_b < (n_a << 5)) { start_b = 0; n_a = 0; }
+  const int n_steps = wave_live ? n_a + ((p_last - start_b) >> 5) + 1 : 0;
+  const int* bt = a.block_table + (long)s * a.bt_stride;
+  const T* kc = (const T*)a.k_cache;
+  const T* vc = (const T*)a.v_cache;
+  const int bs = a.block_size, bs8 = a.block_size >> 3;
+  f32x4 acc[VT];
+#pragma unroll
+  for (int c = 0; c < VT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int lo_row = a.window > 0 ? pos - a.window + 1 : 0;
+  for (int si = wk; si < n_steps; si += kw) {
+    const int base = si < n_a ? (si << 5) : start_b + ((si - n_a) << 5);
+    // K rows of the two interleaved tiles
+    const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
+    const int ka = min(key0, p_last), kb = min(key0 + 4, p_last);
+    const long blk_a = bt[ka / bs], blk_b = bt[kb / bs];
+    const T* kpa = kc + ((blk_a * a.G + g) * bs + (ka % bs)) * (long)D + 8 * g4;
+    const T* kpb = kc + ((blk_b * a.G + g) * bs + (kb % bs)) * (long)D + 8 * g4;
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < DT; ++k) {
+      s0 = mfma16(ld8<T>(kpa + 32 * k), qf[k], s0);
+      s1 = mfma16(ld8<T>(kpb + 32 * k), qf[k], s1);
+    }
+    // V^T rows: this lane's 8 keys are base + 8 * g4 .. + 7, channel 16 * c + r16
+    const int vkey = min(base + 8 * g4, p_last) & ~7;
+    const long blk_v = bt[vkey / bs];
+    const T* vp = vc + (((blk_v * a.G + g) * bs8 + ((vkey % bs) >> 3)) * (long)DV + r16) * 8;
+    V8 vf[VT];
+#pragma unroll
+    for (int c = 0; c < VT; ++c) vf[c] = ld8<T>(vp + (long)c * 128);
+    const int kidx0 = base + 8 * g4;
+    float p[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = kidx0 + j;
+      float sv = (j < 4 ? s0[j & 3] : s1[j & 3]) * scale2;
+      if (a.softcap > 0.f) {
+        const float e = fast_exp2(sv * (2.f / a.softcap));
+        sv = (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e)) * (a.softcap * LOG2E);
+      }
+      // r1 * ln(1 + r2 * dist) on the log2 scale = (r1 ln2 log2e) * log2(1 + r2 * dist); v_log_f32 is log2
+      if (a.bias_scale) sv -= r1 * __builtin_amdgcn_logf(fmaf(r2, (float)max(pos - key, 0), 1.f));
+      const bool seen = row_ok && key <= pos && (key >= lo_row || key < a.keep_first);
+      p[j] = seen ? sv : -INFINITY;
+      tmax = fmaxf(tmax, p[j]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;       // a row with nothing visible yet: every weight 0
+    const float alpha = fast_exp2(m - m_use);                    // (m = -inf: 0)
+    float psum = 0.f;
+    V8 ph, pl;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float e = fast_exp2(p[j] - m_use);                   // (masked: 2^-inf = 0)
+      psum += e;
+      const T hi = (T)e;
+      ph[j] = hi;
+      pl[j] = (T)(e - (float)hi);
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int c = 0; c < VT; ++c) {
+      acc[c] *= alpha;
+      acc[c] = mfma16(vf[c], ph, acc[c]);
+      acc[c] = mfma16(vf[c], pl, acc[c]);
+    }
+  }
+  // ---- merge the key-split waves of a row set (wave wk == 0 of each set ends up with the result)
+  if (kw > 1) {
+    // per (token-wave, key-wave, lane): m, l, VT * 4 accumulators
+    const int per = 2 + 4 * VT;
+    float* mine = lds + ((long)(wt * kw + wk) * 64 + lane) * per;
+    if (wk > 0) {
+      mine[0] = m; mine[1] = l;
+#pragma unroll
+      for (int c = 0; c < VT; ++c) { mine[2 + 4 * c] = acc[c][0]; mine[3 + 4 * c] = acc[c][1]; mine[4 + 4 * c] = acc[c][2]; mine[5 + 4 * c] = acc[c][3]; }
+    }
+    __syncthreads();
+    if (wk > 0) return;
+    for (int o = 1; o < kw; ++o) {
+      const float* th = lds + ((long)(wt * kw + o) * 64 + lane) * per;
+      const float m_o = th[0], l_o = th[1];
+      const float m_new = fmaxf(m, m_o);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float fa = fast_exp2(m - m_use), fb = fast_exp2(m_o - m_use);
+      l = l * fa + l_o * fb;
+      m = m_new;
+#pragma unroll
+      for (int c = 0; c < VT; ++c) {
+        acc[c][0] = acc[c][0] * fa + th[2 + 4 * c] * fb;
+        acc[c][1] = acc[c][1] * fa + th[3 + 4 * c] * fb;
+        acc[c][2] = acc[c][2] * fa + th[4 + 4 * c] * fb;
+        acc[c][3] = acc[c][3] * fa + th[5 + 4 * c] * fb;
+      }
+    }
+  }
+  if (!row_ok) return;
+  if (a.sinks) {
+    const float sk = a.sinks[h] * LOG2E;
+    const float m_f = fmaxf(m, sk);
+    const float fa = fast_exp2(m - m_f);
+    l = l * fa + fast_exp2(sk - m_f);
+#pragma unroll
+    for (int c = 0; c < VT; ++c) acc[c] *= fa;
+  }
+  float mul = 1.0f / l;
+  if (a.gate) {
+    const float gv = (float)((const T*)a.gate)[trow * a.gate_stride + h];
+    mul *= 1.0f / (1.0f + expf(-gv));
+  }
+  T* o = (T*)a.out + (trow * a.H + h) * (long)DV + 4 * g4;
+#pragma unroll
+  for (int c = 0; c < VT; ++c) {
+    bf16x4 ov;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ov[i] = (T)(acc[c][i] * mul);
+    *reinterpret_cast<bf16x4*>(o + 16 * c) = ov;
   }
 }
 
@@ -451,17 +652,61 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
   });
 }
 
+namespace {
+
+template <int DT> int launch_mfma(int vt, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const AttnArgs& a,
+                                  const int* qsl, const int* seq_lens, int hp, int tpw, int kw) {
+  switch (vt) {
+#define VDAMD_CASE(VT_)                                                                                         \
+  case VT_:                                                                                                     \
+    hipLaunchKernelGGL((window_bias_attention_mfma_kernel<DT, VT_>), grid, block, lds, stream, a, qsl, seq_lens, \
+                       hp, tpw, kw);                                                                            \
+    return 0;
+    VDAMD_CASE(1) VDAMD_CASE(2) VDAMD_CASE(4) VDAMD_CASE(8)
+#undef VDAMD_CASE
+  }
+  return 1;
+}
+
+}  // namespace
+
+// q [T, H, D]; sequence b owns rows qsl[b] .. qsl[b + 1], the last positions of its seq_lens[b] tokens
+// (token_seq / positions say the same per row, for the kernel that walks rows).  use_mfma: 0 never, 1 when the
+// shape allows (bf16, D a multiple of 32 up to 256, Dv in {16, 32, 64, 128}).
 VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, const void* v_cache,
                                           const int* block_table, long bt_stride, const int* token_seq,
-                                          const int* positions, const float* bias_scale, const float* bias_rate,
-                                          const float* sinks, const void* gate, long gate_stride, void* out, int T,
-                                          int H, int G, int D, int Dv, int block_size, int window, int keep_first,
-                                          float scale, float softcap, int dt, hipStream_t stream) {
+                                          const int* positions, const int* qsl, const int* seq_lens,
+                                          const float* bias_scale, const float* bias_rate, const float* sinks,
+                                          const void* gate, long gate_stride, void* out, int T, int B, int H, int G,
+                                          int D, int Dv, int block_size, int window, int keep_first,
+                                          int max_query_len, float scale, float softcap, int use_mfma, int dt,
+                                          hipStream_t stream) {
   if (T <= 0) return 0;
-  if (H % G || D <= 0 || Dv <= 0 || Dv > 64 * ATTN_V_PER_LANE || block_size <= 0 || (bias_scale && !bias_rate)) return 1;
+  if (H % G || D <= 0 || Dv <= 0 || Dv > 64 * ATTN_V_PER_LANE || block_size <= 0 || block_size % 8 ||
+      (bias_scale && !bias_rate))
+    return 1;
   AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
              gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap};
   const int qpg = H / G;
+  const int dtiles = D / 32, vtiles = Dv / 16;
+  if (use_mfma && dt == DT_BF16 && qsl && seq_lens && B > 0 && max_query_len > 0 && D % 32 == 0 && Dv % 16 == 0 &&
+      (dtiles == 1 || dtiles == 2 || dtiles == 4 || dtiles == 8) &&
+      (vtiles == 1 || vtiles == 2 || vtiles == 4 || vtiles == 8)) {
+    const int hp = qpg < 16 ? qpg : 16;
+    const int tpw = 16 / hp;
+    const int hchunks = (qpg + hp - 1) / hp;
+    int tw = 4, kw = 1;
+    if (max_query_len <= tpw) { tw = 1; kw = 4; }          // few rows, many keys: the waves share the keys
+    const int gx = (max_query_len + tw * tpw - 1) / (tw * tpw);
+    const size_t lds = kw > 1 ? (size_t)tw * kw * 64 * (2 + 4 * vtiles) * sizeof(float) : 0;
+    const dim3 grid(gx, G * hchunks, B), block(64 * tw * kw);
+    switch (dtiles) {
+      case 1: return launch_mfma<1>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+      case 2: return launch_mfma<2>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+      case 4: return launch_mfma<4>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+      case 8: return launch_mfma<8>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+    }
+  }
   const int waves = qpg < ATTN_MAX_WAVES ? qpg : ATTN_MAX_WAVES;
   const int chunks = (qpg + waves - 1) / waves;
   const size_t lds = (((size_t)waves * (D + 128) + 1) & ~(size_t)1) * sizeof(float) + (size_t)waves * 64 * sizeof(long);

@@ -68,7 +68,7 @@ def _conv_case(dtype, h, g, d, dv, taps, chunks, seed):
     table = torch.randperm(nblocks, device="cuda", generator=gen).to(torch.int32).view(b, -1)
     slot_map = torch.stack([table[s, p // bs] * bs + p % bs for s, p in zip(tok_seq.tolist(), pos.tolist())]).to(torch.int32)
     kc = torch.zeros(nblocks, g, bs, d, device="cuda", dtype=dtype)
-    vc = torch.zeros(nblocks, g, bs, dv, device="cuda", dtype=dtype)
+    vc = torch.zeros(nblocks, g, bs // 8, dv, 8, device="cuda", dtype=dtype)
     qn = torch.rand(d, device="cuda", generator=gen) + 0.5
     kn = torch.rand(d, device="cuda", generator=gen) + 0.5
     vf = torch.randn(n_rows, g * dv, device="cuda", generator=gen)
@@ -126,9 +126,13 @@ def test_conv_decode_rows_own_their_state():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(12, 3, 64, 32), (6, 3, 32, 48), (4, 1, 16, 16), (4, 4, 128, 128), (2, 2, 72, 8),
                                    (40, 2, 64, 64)])
-@pytest.mark.parametrize("window,keep", [(0, 0), (20, 0), (20, 3), (200, 7), (1, 2)])
-def test_window_bias_attention(dtype, shape, window, keep):
+@pytest.mark.parametrize("window,keep", [(0, 0), (20, 0), (20, 3), (200, 7), (1, 2), (40, 70)])
+@pytest.mark.parametrize("mfma", [True, False])
+def test_window_bias_attention(dtype, shape, window, keep, mfma, monkeypatch):
     hip = _hip()
+    if not mfma and dtype != torch.bfloat16:
+        pytest.skip("the plain kernel is the only one for fp32")
+    monkeypatch.setattr(hip, "WINDOW_ATTENTION_MFMA", mfma)
     h, g, d, dv = shape
     gen = torch.Generator(device="cuda").manual_seed(h * 131 + window)
     bs, nblocks = 16, 40
@@ -136,7 +140,7 @@ def test_window_bias_attention(dtype, shape, window, keep):
     b = len(chunks)
     n_rows = sum(n for _, n in chunks)
     kc = torch.randn(nblocks, g, bs, d, device="cuda", generator=gen).to(dtype)
-    vc = torch.randn(nblocks, g, bs, dv, device="cuda", generator=gen).to(dtype)
+    vc = torch.randn(nblocks, g, bs // 8, dv, 8, device="cuda", generator=gen).to(dtype)
     q = torch.randn(n_rows, h, d, device="cuda", generator=gen).to(dtype)
     gate = torch.randn(n_rows, h + 5, device="cuda", generator=gen).to(dtype)[:, 5:]
     table = torch.randint(0, nblocks, (b, 10), device="cuda", generator=gen, dtype=torch.int32)
@@ -150,8 +154,35 @@ def test_window_bias_attention(dtype, shape, window, keep):
     for use_bias, use_sink, use_gate, cap in ((True, True, True, 7.0), (False, False, False, 0.0)):
         got = hip.window_bias_attention(q, kc, vc, table, qsl, seq_lens, tok_seq, pos, 0.2, cap, window, keep,
                                         r1 if use_bias else None, r2 if use_bias else None,
-                                        sink if use_sink else None, gate if use_gate else None)
+                                        sink if use_sink else None, gate if use_gate else None, 70)
         want = torch_ref.window_bias_attention(q, kc, vc, table, qsl, seq_lens, 0.2, cap, window, keep,
                                                r1 if use_bias else None, r2 if use_bias else None,
                                                sink if use_sink else None, gate if use_gate else None)
         _close(got, want, dtype, 4)
+
+
+@pytest.mark.parametrize("shape", [(12, 3, 64, 32), (4, 4, 128, 128), (40, 2, 64, 64), (6, 3, 32, 16), (16, 1, 256, 128)])
+@pytest.mark.parametrize("window,keep", [(0, 0), (33, 5), (700, 40)])
+def test_window_bias_attention_decode_rows(shape, window, keep):
+    """One row per sequence (no row map, the waves of a block share the keys), contexts from 1 to 900 keys."""
+    hip = _hip()
+    h, g, d, dv = shape
+    dtype = torch.bfloat16
+    gen = torch.Generator(device="cuda").manual_seed(h + window)
+    bs, nblocks = 16, 80
+    lens = [1, 2, 31, 32, 33, 64, 257, 900]
+    b = len(lens)
+    kc = torch.randn(nblocks, g, bs, d, device="cuda", generator=gen).to(dtype)
+    vc = torch.randn(nblocks, g, bs // 8, dv, 8, device="cuda", generator=gen).to(dtype)
+    q = torch.randn(b, h, d, device="cuda", generator=gen).to(dtype)
+    gate = torch.randn(b, h, device="cuda", generator=gen).to(dtype)
+    table = torch.randint(0, nblocks, (b, 60), device="cuda", generator=gen, dtype=torch.int32)
+    qsl = torch.arange(b + 1, dtype=torch.int32, device="cuda")
+    seq_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    pos = seq_lens - 1
+    r1 = torch.rand(h, device="cuda", generator=gen)
+    r2 = torch.rand(h, device="cuda", generator=gen)
+    sink = torch.randn(h, device="cuda", generator=gen)
+    got = hip.window_bias_attention(q, kc, vc, table, qsl, seq_lens, None, pos, 0.2, 9.0, window, keep, r1, r2, sink, gate, 1)
+    want = torch_ref.window_bias_attention(q, kc, vc, table, qsl, seq_lens, 0.2, 9.0, window, keep, r1, r2, sink, gate)
+    _close(got, want, dtype, 4)

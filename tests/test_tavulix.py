@@ -268,9 +268,9 @@ def _attention_case(device, dtype, n, d, dv, bs=16):
     table = torch.randperm(nblocks, generator=g)[:-(-n // bs)].to(torch.int32).view(1, -1)
     keys = torch.randn(n, d, generator=g) * 0.05
     vals = torch.randn(n, dv, generator=g)
-    kc, vc = torch.zeros(nblocks, 1, bs, d), torch.zeros(nblocks, 1, bs, dv)
+    kc, vc = torch.zeros(nblocks, 1, bs, d), torch.zeros(nblocks, 1, bs // 8, dv, 8)
     for j in range(n):
-        kc[table[0, j // bs], 0, j % bs], vc[table[0, j // bs], 0, j % bs] = keys[j], vals[j]
+        kc[table[0, j // bs], 0, j % bs], vc[table[0, j // bs], 0, (j % bs) // 8, :, j % 8] = keys[j], vals[j]
     to = lambda t: t.to(device)                                           # noqa: E731
     return keys, vals, to(kc.to(dt)), to(vc.to(dt)), to(table)
 
@@ -312,9 +312,9 @@ def test_sink_cap_and_distance_bias_show(device, dtype, tol):
     from vllm_distributed_amd import ops
     d, dv = 16, 8
     dt = getattr(torch, dtype)
-    kc, vc = torch.zeros(2, 1, 16, d), torch.zeros(2, 1, 16, dv)
+    kc, vc = torch.zeros(2, 1, 16, d), torch.zeros(2, 1, 2, dv, 8)
     kc[1, 0, :, 0] = 1.0
-    vc[1, 0, :, :] = 1.0
+    vc[1] = 1.0
     table = torch.tensor([[1, 0]], dtype=torch.int32, device=device)
     for pos, window, sink, cap, r1, r2, raw in ((0, 4, 0.7, 2.0, 0.5, 0.3, 5.0), (3, 1, -1.5, 0.0, 0.9, 2.0, 1.0),
                                                 (3, 1, 30.0, 1.0, 0.0, 0.0, 0.4)):
@@ -332,7 +332,7 @@ def test_sink_cap_and_distance_bias_show(device, dtype, tol):
     # two visible keys at distances 0 and 1 with equal raw scores: the bias alone decides their weights
     q = torch.zeros(1, 1, d)
     vc2 = vc.clone()
-    vc2[1, 0, 0, :] = 0.0                                   # key 0 carries value 0, key 1 value 1
+    vc2[1, 0, 0, :, 0] = 0.0                                # key 0 carries value 0, key 1 value 1
     out = ops.window_bias_attention(
         q.to(dt).to(device), kc.to(dt).to(device), vc2.to(dt).to(device), table,
         torch.tensor([0, 1], dtype=torch.int32, device=device), torch.tensor([2], dtype=torch.int32, device=device),

@@ -210,8 +210,8 @@ class WindowBiasAttention(Attention):
     a rotation, an optional score cap, a sink in the softmax denominator and a sigmoid gate on each head's output;
     key and value heads may differ in size.  A query at position ``i`` sees key ``j <= i`` when
     ``i - j < window`` or ``j < keep_first``; its score is ``cap(q.k * scale) - bias_scale[h] * ln(1 +
-    bias_rate[h] * (i - j))``.  The caches are plain rows, ``[blocks, Hkv, block, dim]`` and ``[blocks, Hkv,
-    block, vdim]``, written by ``ops.conv_norm_cache`` (this layer's callers convolve and normalise q / k / v
+    bias_rate[h] * (i - j))``.  The caches are key rows ``[blocks, Hkv, block, dim]`` and values with eight keys side
+    by side per channel, ``[blocks, Hkv, block / 8, vdim, 8]``, written by ``ops.conv_norm_cache`` (this layer's callers convolve and normalise q / k / v
     first); scores, softmax and the weighted sum of values are fp32 in every dtype."""
     row_cache = True
 
@@ -228,8 +228,10 @@ class WindowBiasAttention(Attention):
         self.sink = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if sink else None
 
     def kv_cache_shapes(self, num_blocks: int, block_size: int):
+        if block_size % 8:
+            raise ValueError("block_size must be a multiple of 8")
         return ((num_blocks, self.num_kv_heads, block_size, self.head_dim),
-                (num_blocks, self.num_kv_heads, block_size, self.vdim))
+                (num_blocks, self.num_kv_heads, block_size // 8, self.vdim, 8))
 
     def kv_values_per_token(self) -> int:
         return self.num_kv_heads * (self.head_dim + self.vdim)

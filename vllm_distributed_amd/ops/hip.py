@@ -68,7 +68,7 @@ def load() -> ctypes.CDLL:
         "vdamd_scalar_norm_residual": [P, P, P, P, P, F, I, I, L, I, I, P],
         "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
         "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, I, P],
-        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, L, P] + [I] * 8 + [F, F, I, P],
+        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, P],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -1263,6 +1263,8 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
 
 CONV_MAX_TAPS = 8
 UNIT_MAX_WIDTH = 512
+# the matrix-core attention kernel where the shape allows it (tests switch it off to run the plain kernel in bf16)
+WINDOW_ATTENTION_MFMA = os.environ.get("VDAMD_WINDOW_ATTENTION_MFMA", "1") != "0"
 
 
 def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
@@ -1286,8 +1288,8 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
     if k_cache is not None:
         bs = k_cache.shape[2]
         assert k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
-        assert k_cache.shape[1:] == (num_kv_heads, bs, dim) and v_cache.shape[1:] == (num_kv_heads, bs, vdim)
-        assert v_cache.shape[0] == k_cache.shape[0]
+        assert k_cache.shape[1:] == (num_kv_heads, bs, dim) and bs % 8 == 0
+        assert v_cache.shape == (k_cache.shape[0], num_kv_heads, bs // 8, vdim, 8)
     else:
         bs = 1
     gv = num_kv_heads * vdim
@@ -1312,9 +1314,11 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
                           gate, max_query_len: int = 0):
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    b = seq_lens.shape[0]
     assert q.is_contiguous() and q.dtype == k_cache.dtype == v_cache.dtype and h % g == 0
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[3] == d
-    assert v_cache.shape[:3] == k_cache.shape[:3] and dv <= UNIT_MAX_WIDTH
+    assert v_cache.shape == (k_cache.shape[0], g, bs // 8, dv, 8) and bs % 8 == 0 and dv <= UNIT_MAX_WIDTH
+    assert query_start_loc.shape[0] >= b + 1 and block_table.shape[0] >= b
     assert block_table.dim() == 2 and block_table.stride(1) == 1 and block_table.dtype == torch.int32
     assert positions.shape[0] >= t and (token_seq is None or token_seq.shape[0] >= t)
     assert token_seq is not None or t <= block_table.shape[0], "rows without a sequence"
@@ -1326,7 +1330,9 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
     _check(_LIB.vdamd_window_bias_attention(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
+        _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(),
         _ptr(_f32_vec(bias_scale, h, "bias_scale")), _ptr(_f32_vec(bias_rate, h, "bias_rate")),
-        _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, h, g, d, dv, bs,
-        int(window), int(keep_first), float(scale), float(softcap), _dt(q), _stream()), "window_bias_attention")
+        _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, b, h, g, d, dv, bs,
+        int(window), int(keep_first), int(max_query_len) if max_query_len else t, float(scale), float(softcap),
+        1 if WINDOW_ATTENTION_MFMA else 0, _dt(q), _stream()), "window_bias_attention")
     return out

@@ -530,7 +530,7 @@ def conv_norm_cache(x: torch.Tensor, conv_weight: torch.Tensor, state: torch.Ten
         sm = slot_mapping[:t][valid].long()
         blk, off = sm // bs, sm % bs
         k_cache[blk, :, off, :] = k[valid].to(k_cache.dtype)
-        v_cache[blk, :, off, :] = v[valid].to(v_cache.dtype)
+        v_cache[blk, :, off // V_GROUP, :, off % V_GROUP] = v[valid].to(v_cache.dtype)
     return q, kept
 
 
@@ -539,7 +539,8 @@ def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           window: int, keep_first: int, bias_scale: Optional[torch.Tensor],
                           bias_rate: Optional[torch.Tensor], sinks: Optional[torch.Tensor],
                           gate: Optional[torch.Tensor]) -> torch.Tensor:
-    """Causal attention over row caches ``k_cache[blocks, Hkv, block, D]`` / ``v_cache[blocks, Hkv, block, Dv]``.
+    """Causal attention over ``k_cache[blocks, Hkv, block, D]`` (key rows) and ``v_cache[blocks, Hkv, block / 8, Dv,
+    8]`` (eight keys side by side per channel).
     A query at position ``i`` sees key ``j <= i`` when ``i - j < window`` (``window`` 0: no limit) or
     ``j < keep_first``.  ``score = q.k * scale``, squashed to ``softcap * tanh(score / softcap)`` when
     ``softcap > 0``, minus ``bias_scale[h] * ln(1 + bias_rate[h] * (i - j))``; ``sinks[h]`` adds ``exp(sinks[h])``
@@ -557,7 +558,7 @@ def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
             continue
         blocks = block_table[i, :(sl + bs - 1) // bs].long()
         k = k_cache[blocks].permute(1, 0, 2, 3).reshape(hkv, -1, d)[:, :sl].float().repeat_interleave(g, dim=0)
-        v = v_cache[blocks].permute(1, 0, 2, 3).reshape(hkv, -1, dv)[:, :sl].float().repeat_interleave(g, dim=0)
+        v = v_cache[blocks].permute(1, 0, 2, 4, 3).reshape(hkv, -1, dv)[:, :sl].float().repeat_interleave(g, dim=0)
         qi = q[s:e].float().transpose(0, 1)
         sc = torch.matmul(qi, k.transpose(1, 2)) * scale
         if softcap > 0:
