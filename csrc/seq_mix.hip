@@ -214,6 +214,114 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
   }
 }
 
+
+// The same for 16-bit types with head sizes that are multiples of 8: a lane owns 8 consecutive channels (16-byte
+// loads and stores), a unit (one head of q, k or v) takes width / 8 lanes, and a wave carries as many units as fit
+// when that is a power of two (the per-head sum of squares is then a few xor-shuffles inside the lane group).
+// Wave tasks are numbered (token, task) across the grid: q and k units first, then v units.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, int gs_d, int upw_d, int gs_v, int upw_v,
+                                                                  int tasks_d, int tasks_v) {
+  using V8 = typename Vec8<T>::type;
+  const int lane = threadIdx.x & 63;
+  const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int tasks = tasks_d + tasks_v;
+  const int t = (int)(wid / tasks);
+  if (t >= a.T) return;
+  const int task = (int)(wid % tasks);
+  const bool is_v = task >= tasks_d;
+  const int gs = is_v ? gs_v : gs_d, upw = is_v ? upw_v : upw_d;
+  const int sub = lane / gs;                      // unit within the wave
+  const int li = lane % gs;                       // lane within the unit
+  const int unit = (is_v ? task - tasks_d : task) * upw + sub;
+  const int n_units = is_v ? a.G : a.H + a.G;
+  const bool live = sub < upw && unit < n_units;
+  int kind, head, width, c0;
+  if (is_v) { kind = 2; head = unit; width = a.Dv; c0 = (a.H + a.G) * a.D + head * a.Dv; }
+  else if (unit < a.H) { kind = 0; head = unit; width = a.D; c0 = unit * a.D; }
+  else { kind = 1; head = unit - a.H; width = a.D; c0 = a.H * a.D + head * a.D; }
+  const int s = a.token_seq ? a.token_seq[t] : t;
+  const int n = a.qsl[s + 1] - a.qsl[s];
+  const int pos = a.positions[t];
+  const int chunk_start = a.seq_lens[s] - n;
+  const int R = a.taps - 1;
+  const int C = a.H * a.D + a.G * (a.D + a.Dv);
+  const T* x = (const T*)a.x;
+  const T* w = (const T*)a.conv_w;
+  T* st = (T*)a.state + (long)a.slots[s] * (R > 0 ? R : 1) * C;
+  const bool own_state = (n == 1) && R > 0;
+  const int c = c0 + 8 * li;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (live) {
+    // the taps of 8 channels are 8 * taps consecutive values
+    const T* wp = w + (long)c * a.taps;
+    for (int j = 0; j < a.taps; ++j) {
+      const int back = a.taps - 1 - j;
+      const int p = pos - back;
+      V8 u;
+      if (p >= chunk_start && p >= 0) u = ld8<T>(x + (long)(t - back) * a.x_stride + c);
+      else if (p >= 0) u = ld8<T>(st + (long)(R - (chunk_start - p)) * C + c);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = (T)0.f;
+      }
+      if (own_state && j >= 1) st8<T>(st + (long)(j - 1) * C + c, u);     // (row j - 1 was read one turn earlier)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)wp[e * a.taps + j] * (float)u[e];
+    }
+  }
+  if (kind < 2) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += acc[e] * acc[e];
+    if (upw == 1) ss = wave_sum(ss);
+    else for (int o = gs >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float inv = 1.0f / sqrtf(ss / (float)width + a.eps);
+    if (live) {
+      const float* nw = (kind == 0 ? a.q_norm : a.k_norm) + 8 * li;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * inv * nw[e];
+    }
+  }
+  if (!live) return;
+  if (kind == 0) {
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (T)acc[e];
+    st8<T>((T*)a.q_out + ((long)t * a.H + head) * a.D + 8 * li, o);
+    return;
+  }
+  if (kind == 2) {
+    const long vrow = (long)t * a.G * a.Dv + (long)head * a.Dv + 8 * li;
+    if (a.v_keep) {
+      *reinterpret_cast<f32x4*>(a.v_keep + vrow) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+      *reinterpret_cast<f32x4*>(a.v_keep + vrow + 4) = f32x4{acc[4], acc[5], acc[6], acc[7]};
+    }
+    if (a.v_first) {
+      const float lam = a.v_lambda[0];
+      const f32x4 f0 = *reinterpret_cast<const f32x4*>(a.v_first + vrow);
+      const f32x4 f1 = *reinterpret_cast<const f32x4*>(a.v_first + vrow + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = (1.0f - lam) * acc[e] + lam * (e < 4 ? f0[e & 3] : f1[e & 3]);
+    }
+  }
+  const int slot = a.slot_mapping[t];
+  if (slot < 0 || a.k_cache == nullptr) return;
+  const long blk = slot / a.block_size, off = slot % a.block_size;
+  if (kind == 1) {
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (T)acc[e];
+    st8<T>((T*)a.k_cache + ((blk * a.G + head) * a.block_size + off) * (long)width + 8 * li, o);
+  } else {                                        // [blocks, G, bs / 8, Dv, 8]: one key's column of 8 channels
+    T* dst = (T*)a.v_cache + (((blk * a.G + head) * (a.block_size >> 3) + (off >> 3)) * (long)width + 8 * li) * 8 + (off & 7);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[e * 8] = (T)acc[e];
+  }
+}
+
 // Sequences that ran two or more rows: their slot takes the last R inputs of (old state ++ this step's rows).
 // One thread per (sequence, channel) reads all R before it writes any.
 template <typename T>
@@ -643,9 +751,26 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
   const int units = H + 2 * G;
   const int waves = units >= 4 ? 4 : units;
   const int C = H * D + G * (D + Dv), R = taps - 1;
+  const bool vec = dt != DT_F32 && D % 8 == 0 && Dv % 8 == 0 && D <= 512 && Dv <= 512 && x_stride % 8 == 0;
+  auto pack = [](int width, int& gs, int& upw) {        // lanes per unit, units per wave
+    gs = width / 8;
+    upw = (gs & (gs - 1)) == 0 ? 64 / gs : 1;
+  };
   return by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
-    hipLaunchKernelGGL((conv_norm_cache_kernel<TT>), dim3(T), dim3(64 * waves), 0, stream, a);
+    if constexpr (!std::is_same_v<TT, float>) {
+      if (vec) {
+        int gs_d, upw_d, gs_v, upw_v;
+        pack(D, gs_d, upw_d);
+        pack(Dv, gs_v, upw_v);
+        const int tasks_d = (H + G + upw_d - 1) / upw_d, tasks_v = (G + upw_v - 1) / upw_v;
+        const long wtasks = (long)T * (tasks_d + tasks_v);
+        hipLaunchKernelGGL((conv_norm_cache_vec_kernel<TT>), dim3((unsigned)((wtasks + 3) / 4)), dim3(256), 0, stream, a,
+                           gs_d, upw_d, gs_v, upw_v, tasks_d, tasks_v);
+      }
+    }
+    if (!vec || std::is_same_v<TT, float>)
+      hipLaunchKernelGGL((conv_norm_cache_kernel<TT>), dim3(T), dim3(64 * waves), 0, stream, a);
     if (update_multi && R > 0)
       hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3((C + 255) / 256, B), dim3(256), 0, stream,
                          (const TT*)x, x_stride, (TT*)state, slots, qsl, C, R);

@@ -57,7 +57,7 @@ def _conv_case(dtype, h, g, d, dv, taps, chunks, seed):
     bs, nblocks = 16, 64
     b = len(chunks)
     n_rows = sum(n for _, n in chunks)
-    x = torch.randn(n_rows, c + h, device="cuda", generator=gen).to(dtype)
+    x = torch.randn(n_rows, c + (8 if seed % 2 else h), device="cuda", generator=gen).to(dtype)
     w = torch.randn(c, taps, device="cuda", generator=gen).to(dtype)
     state = torch.randn(b + 2, max(taps - 1, 1), c, device="cuda", generator=gen).to(dtype)
     slots = torch.randperm(b + 2, device="cuda", generator=gen)[:b].to(torch.int32)

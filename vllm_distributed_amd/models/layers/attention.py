@@ -55,6 +55,19 @@ class AttentionMetadata:
         return cached
 
 
+def _prefill_token_rows(self, positions: torch.Tensor) -> torch.Tensor:
+    """For the prompt-chunk rows of the step (those behind the decode rows): the sequence each belongs to, counted
+    from the first prefill sequence; computed once per step and kept."""
+    cached = getattr(self, "_prefill_rows", None)
+    if cached is None:
+        rows = self.token_rows(positions)[0]
+        cached = self._prefill_rows = (rows[self.num_decode_tokens:] - self.num_decodes).contiguous()
+    return cached
+
+
+AttentionMetadata.prefill_token_rows = _prefill_token_rows
+
+
 class ForwardContext:
     attn_metadata: Optional[AttentionMetadata] = None
     positions: Optional[torch.Tensor] = None
@@ -242,10 +255,19 @@ class WindowBiasAttention(Attention):
         t = q.shape[0]
         if md is None:               # memory-profiling pass: no cache bound
             return q.new_zeros((t, self.num_heads * self.vdim))
-        rows = None if md.num_prefills == 0 else md.token_rows(_CTX.positions)[0]
-        out = ops.window_bias_attention(q, self.k_cache, self.v_cache, md.block_table, md.query_start_loc, md.seq_lens,
-                                        rows, _CTX.positions, self.scale, self.softcap, self.window, self.keep_first,
-                                        self.bias_scale, self.bias_rate, self.sink, gate, md.max_query_len)
+        out = torch.empty((t, self.num_heads, self.vdim), dtype=q.dtype, device=q.device)
+        pos = _CTX.positions
+        nd, nb = md.num_decode_tokens, md.num_decodes
+        common = (self.scale, self.softcap, self.window, self.keep_first, self.bias_scale, self.bias_rate, self.sink)
+        if nd > 0:            # one row per sequence: the waves of a block share its keys
+            ops.window_bias_attention(q[:nd], self.k_cache, self.v_cache, md.block_table[:nb], md.query_start_loc[:nb + 1],
+                                      md.seq_lens[:nb], None, pos[:nd], *common,
+                                      None if gate is None else gate[:nd], 1, out=out[:nd])
+        if md.num_prefills > 0:
+            ops.window_bias_attention(q[nd:], self.k_cache, self.v_cache, md.block_table[nb:],
+                                      md.prefill_query_start_loc, md.seq_lens[nb:], md.prefill_token_rows(pos), pos[nd:],
+                                      *common, None if gate is None else gate[nd:], md.max_prefill_query_len,
+                                      out=out[nd:])
         return out.view(t, self.num_heads * self.vdim)
 
 

@@ -655,13 +655,17 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
 
 def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
                           scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
-                          gate, max_query_len: int = 0):
+                          gate, max_query_len: int = 0, out=None):
     """Attention over row caches with a window that keeps the first keys, a logarithmic distance bias, a sink in
     the denominator and an output gate; see ``torch_ref.window_bias_attention``."""
     if _use_hip(q):
         attention_calls["hip"] += 1
         return _hip.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq,
                                           positions, scale, softcap, window, keep_first, bias_scale, bias_rate, sinks,
-                                          gate, max_query_len)
-    return torch_ref.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, scale,
-                                           softcap, window, keep_first, bias_scale, bias_rate, sinks, gate)
+                                          gate, max_query_len, out)
+    res = torch_ref.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, scale,
+                                          softcap, window, keep_first, bias_scale, bias_rate, sinks, gate)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res

@@ -1311,7 +1311,7 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
 
 def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
                           scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
-                          gate, max_query_len: int = 0):
+                          gate, max_query_len: int = 0, out=None):
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     b = seq_lens.shape[0]
@@ -1326,7 +1326,9 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
     if gate is not None:
         assert gate.shape == (t, h) and gate.stride(1) == 1 and gate.dtype == q.dtype
         gate_stride = gate.stride(0)
-    out = torch.empty((t, h, dv), dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((t, h, dv), dtype=q.dtype, device=q.device)
+    assert out.shape == (t, h, dv) and out.dtype == q.dtype and out.is_contiguous()
     _check(_LIB.vdamd_window_bias_attention(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
