@@ -27,6 +27,19 @@ namespace {
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)(*p); }
 template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
 
+// residual stream at its start: token row + position row, summed in fp32
+template <typename T>
+__global__ void embed_positions_kernel(float* __restrict__ out, const int* __restrict__ ids,
+                                       const int* __restrict__ positions, const T* __restrict__ embed,
+                                       const T* __restrict__ pos, int H, int vocab_rows, int pos_rows) {
+  const long t = blockIdx.x;
+  const int id = min(max(ids[t], 0), vocab_rows - 1), p = min(max(positions[t], 0), pos_rows - 1);
+  const T* e = embed + (long)id * H;
+  const T* q = pos + (long)p * H;
+  float* o = out + t * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ldf(e + i) + ldf(q + i);
+}
+
 // ------------------------------------------------------------------------------------------------ norms
 template <typename TI, typename TO>
 __global__ void scalar_norm_kernel(TO* __restrict__ out, const TI* __restrict__ x, const float* __restrict__ gain,
@@ -93,7 +106,7 @@ __global__ void poly_norm_kernel(T* __restrict__ out, const T* __restrict__ z, c
 }
 
 // ---------------------------------------------------------------------------- convolution + norm + cache write
-constexpr int CONV_MAX_TAPS = 8;
+constexpr int CONV_MAX_TAPS = 16;
 constexpr int UNIT_MAX_PER_LANE = 8;        // a head is at most 64 * 8 = 512 channels wide
 
 struct ConvArgs {
@@ -687,6 +700,17 @@ template <typename F> int by_dtype(int dt, F&& f) {
 int norm_threads(int h) { return h >= 2048 ? 512 : (h >= 512 ? 256 : 128); }
 
 }  // namespace
+
+VDAMD_API int vdamd_embed_positions(float* out, const int* ids, const int* positions, const void* embed, const void* pos,
+                                    int T, int H, int vocab_rows, int pos_rows, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || vocab_rows <= 0 || pos_rows <= 0) return 1;
+  return by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((embed_positions_kernel<TT>), dim3(T), dim3(norm_threads(H)), 0, stream, out, ids, positions,
+                       (const TT*)embed, (const TT*)pos, H, vocab_rows, pos_rows);
+  });
+}
 
 // out[rows, H] (dtype out_dt) = x[rows, x_stride..] (dtype in_dt) normalised with one gain
 VDAMD_API int vdamd_scalar_norm(void* out, const void* x, const float* gain, float eps, int rows, int H, long x_stride,

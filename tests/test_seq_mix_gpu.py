@@ -186,3 +186,17 @@ def test_window_bias_attention_decode_rows(shape, window, keep):
     got = hip.window_bias_attention(q, kc, vc, table, qsl, seq_lens, None, pos, 0.2, 9.0, window, keep, r1, r2, sink, gate, 1)
     want = torch_ref.window_bias_attention(q, kc, vc, table, qsl, seq_lens, 0.2, 9.0, window, keep, r1, r2, sink, gate)
     _close(got, want, dtype, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("h", [8, 37, 256])
+def test_embed_positions(dtype, h):
+    hip = _hip()
+    g = torch.Generator(device="cuda").manual_seed(h)
+    emb = torch.randn(50, h, device="cuda", generator=g).to(dtype)
+    pos = torch.randn(30, h, device="cuda", generator=g).to(dtype)
+    ids = torch.randint(0, 50, (40,), device="cuda", generator=g, dtype=torch.int32)
+    ps = torch.randint(0, 30, (40,), device="cuda", generator=g, dtype=torch.int32)
+    got = hip.embed_positions(ids, ps, emb, pos)
+    assert got.dtype == torch.float32
+    assert torch.equal(got, emb[ids.long()].float() + pos[ps.long()].float())

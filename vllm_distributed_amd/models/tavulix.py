@@ -155,7 +155,7 @@ class TavulixForCausalLM(nn.Module):
         return [l.mix.conv for l in self.layers]
 
     def forward(self, input_ids, positions, intermediate: Optional[IntermediateTensors] = None):
-        x = self.embed(input_ids).float() + self.pos(positions.long()).float()
+        x = ops.embed_positions(input_ids, positions, self.embed.weight, self.pos.weight)
         n = len(self.layers)
         h = self.layers[0].norm1(x) if n else None
         v_first = None

@@ -617,6 +617,13 @@ def mla_prep(q, nope, q_lat, latent, norm_weight, eps, cos_sin, positions, k_cac
 
 
 # ------------------------------------------------ single-gain norms, PolyNorm, convolved q/k/v, windowed attention
+def embed_positions(ids, positions, embed, pos):
+    """``embed[ids] + pos[positions]`` summed in fp32: the residual stream of a model with learned positions."""
+    if _use_hip(embed):
+        return _hip.embed_positions(ids, positions, embed, pos)
+    return embed[ids.long()].float() + pos[positions.long()].float()
+
+
 def scalar_rms_norm(x, gain, eps: float, out_dtype):
     """RMS norm with one gain for the whole row (fp32 arithmetic), result in ``out_dtype``."""
     if _use_hip(x):

@@ -64,6 +64,7 @@ def load() -> ctypes.CDLL:
         "vdamd_fp4a16_gemm": [P, L, P, L, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_fp4_dequant": [P, P, P, P, I, I, I, P],
         "vdamd_fp4a16_gemm_grouped": [P, L, P, L, P, P, L, L, P, P, I, I, I, I, I, P],
+        "vdamd_embed_positions": [P, P, P, P, P, I, I, I, I, I, P],
         "vdamd_scalar_norm": [P, P, P, F, I, I, L, I, I, P],
         "vdamd_scalar_norm_residual": [P, P, P, P, P, F, I, I, L, I, I, P],
         "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
@@ -1227,6 +1228,19 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+def embed_positions(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+    t, h = ids.shape[0], embed.shape[1]
+    assert ids.dim() == 1 and positions.shape[0] >= t and embed.is_contiguous() and pos.is_contiguous()
+    assert pos.shape[1] == h and pos.dtype == embed.dtype
+    ids = ids if ids.dtype == torch.int32 else ids.to(torch.int32)
+    positions = positions if positions.dtype == torch.int32 else positions.to(torch.int32)
+    out = torch.empty((t, h), dtype=torch.float32, device=embed.device)
+    _check(_LIB.vdamd_embed_positions(out.data_ptr(), _i32(ids, "ids").data_ptr(), _i32(positions, "positions").data_ptr(),
+                                      embed.data_ptr(), pos.data_ptr(), t, h, embed.shape[0], pos.shape[0], _dt(embed),
+                                      _stream()), "embed_positions")
+    return out
+
+
 def scalar_rms_norm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
     h = x.shape[-1]
     x2 = x.reshape(-1, h)
@@ -1261,7 +1275,7 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
     return out.view(z.shape)
 
 
-CONV_MAX_TAPS = 8
+CONV_MAX_TAPS = 16
 UNIT_MAX_WIDTH = 512
 # the matrix-core attention kernel where the shape allows it (tests switch it off to run the plain kernel in bf16)
 WINDOW_ATTENTION_MFMA = os.environ.get("VDAMD_WINDOW_ATTENTION_MFMA", "1") != "0"
