@@ -571,8 +571,17 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   for (int c = 0; c < VT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int lo_row = a.window > 0 ? pos - a.window + 1 : 0;
-  for (int si = wk; si < n_steps; si += kw) {
+  // a step all of whose 32 keys every row of the wave sees needs no mask: inside [window start of the wave's
+  // last row, position of its first row], or inside the kept first keys
+  const int full_lo = a.window > 0 ? p_last - a.window + 1 : 0;
+  const float posf = (float)pos;
+  const float cap_in = a.softcap > 0.f ? 2.f / a.softcap : 0.f, cap_out = a.softcap * LOG2E;
+  // newest keys first: with a distance bias they carry the largest scores, so the running maximum settles in the
+  // first steps and the accumulators are rarely rescaled afterwards
+  for (int it = wk; it < n_steps; it += kw) {
+    const int si = n_steps - 1 - it;
     const int base = si < n_a ? (si << 5) : start_b + ((si - n_a) << 5);
+    const bool interior = base + 31 <= p_first && (base >= full_lo || base + 31 < a.keep_first);
     // K rows of the two interleaved tiles
     const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
     const int ka = min(key0, p_last), kb = min(key0 + 4, p_last);
@@ -593,22 +602,28 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
 #pragma unroll
     for (int c = 0; c < VT; ++c) vf[c] = ld8<T>(vp + (long)c * 128);
     const int kidx0 = base + 8 * g4;
+    const float d0 = posf - (float)kidx0;          // distance of this lane's key j: d0 - j
     float p[8];
-    float tmax = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int key = kidx0 + j;
       float sv = (j < 4 ? s0[j & 3] : s1[j & 3]) * scale2;
-      if (a.softcap > 0.f) {
-        const float e = fast_exp2(sv * (2.f / a.softcap));
-        sv = (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e)) * (a.softcap * LOG2E);
+      if (a.softcap > 0.f) {                       // cap * tanh(s / cap) = cap * (1 - 2 / (1 + e^(2 s / cap)))
+        const float e = fast_exp2(sv * cap_in);
+        sv = fmaf(-2.f * cap_out, __builtin_amdgcn_rcpf(1.f + e), cap_out);
       }
-      // r1 * ln(1 + r2 * dist) on the log2 scale = (r1 ln2 log2e) * log2(1 + r2 * dist); v_log_f32 is log2
-      if (a.bias_scale) sv -= r1 * __builtin_amdgcn_logf(fmaf(r2, (float)max(pos - key, 0), 1.f));
-      const bool seen = row_ok && key <= pos && (key >= lo_row || key < a.keep_first);
-      p[j] = seen ? sv : -INFINITY;
-      tmax = fmaxf(tmax, p[j]);
+      // r1 * ln(1 + r2 * dist) on the log2 scale is r1 * log2(1 + r2 * dist); v_log_f32 is log2
+      if (a.bias_scale) sv = fmaf(-r1, __builtin_amdgcn_logf(fmaf(r2, d0 - (float)j, 1.f)), sv);
+      p[j] = sv;
     }
+    if (!interior) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = kidx0 + j;
+        const bool seen = row_ok && key <= pos && (key >= lo_row || key < a.keep_first);
+        p[j] = seen ? p[j] : -INFINITY;            // (also drops the NaN a negative distance gives the logarithm)
+      }
+    }
+    float tmax = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(m, tmax);
@@ -628,9 +643,12 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     psum += __shfl_xor(psum, 32, 64);
     l = l * alpha + psum;
     m = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int c = 0; c < VT; ++c) acc[c] *= alpha;
+    }
 #pragma unroll
     for (int c = 0; c < VT; ++c) {
-      acc[c] *= alpha;
       acc[c] = mfma16(vf[c], ph, acc[c]);
       acc[c] = mfma16(vf[c], pl, acc[c]);
     }
