@@ -105,13 +105,95 @@ __global__ void poly_norm_kernel(T* __restrict__ out, const T* __restrict__ z, c
   }
 }
 
+
+// 16-bit rows whose length and stride are multiples of 8: the same two kernels with 16-byte accesses
+template <typename T>
+__global__ void poly_norm_vec_kernel(T* __restrict__ out, const T* __restrict__ z, const float* __restrict__ coef,
+                                     float eps, int F, long z_stride) {
+  using V8 = typename Vec8<T>::type;
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const T* zr = z + row * z_stride;
+  const int nv = F >> 3;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const V8 v = ld8<T>(zr + 8 * i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)v[e], f2 = f * f, f3 = f2 * f;
+      s2 += f2; s4 += f2 * f2; s6 += f3 * f3;
+    }
+  }
+  s2 = block_sum(s2, red);
+  s4 = block_sum(s4, red);
+  s6 = block_sum(s6, red);
+  const float n = (float)F;
+  const float a = coef[0] / sqrtf(s2 / n + eps), b = coef[1] / sqrtf(s4 / n + eps), c = coef[2] / sqrtf(s6 / n + eps);
+  const float e0 = coef[3];
+  T* orow = out + row * (long)F;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const V8 v = ld8<T>(zr + 8 * i);
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)v[e], f2 = f * f;
+      o[e] = (T)(a * f + b * f2 + c * f2 * f + e0);
+    }
+    st8<T>(orow + 8 * i, o);
+  }
+}
+
+template <typename T>
+__global__ void scalar_norm_residual_vec_kernel(T* __restrict__ out, const T* __restrict__ y, float* __restrict__ residual,
+                                                const float* __restrict__ g_post, const float* __restrict__ g_next,
+                                                float eps, int H, long y_stride) {
+  using V8 = typename Vec8<T>::type;
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float* rr = residual + row * (long)H;
+  const int nv = H >> 3;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const V8 v = ld8<T>(yr + 8 * i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; ss += f * f; }
+  }
+  ss = block_sum(ss, red);
+  const float inv = (1.0f / sqrtf(ss / (float)H + eps)) * g_post[0];
+  float s2 = 0.f;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const V8 v = ld8<T>(yr + 8 * i);
+    f32x4 r0 = *reinterpret_cast<const f32x4*>(rr + 8 * i), r1 = *reinterpret_cast<const f32x4*>(rr + 8 * i + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r0[e] += (float)v[e] * inv;
+      r1[e] += (float)v[e + 4] * inv;
+      s2 += r0[e] * r0[e] + r1[e] * r1[e];
+    }
+    *reinterpret_cast<f32x4*>(rr + 8 * i) = r0;
+    *reinterpret_cast<f32x4*>(rr + 8 * i + 4) = r1;
+  }
+  if (out == nullptr) return;
+  s2 = block_sum(s2, red);
+  const float inv2 = (1.0f / sqrtf(s2 / (float)H + eps)) * g_next[0];
+  T* orow = out + row * (long)H;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {                 // (each thread rereads its own stores)
+    const f32x4 r0 = *reinterpret_cast<const f32x4*>(rr + 8 * i), r1 = *reinterpret_cast<const f32x4*>(rr + 8 * i + 4);
+    V8 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { o[e] = (T)(r0[e] * inv2); o[e + 4] = (T)(r1[e] * inv2); }
+    st8<T>(orow + 8 * i, o);
+  }
+}
+
 // ---------------------------------------------------------------------------- convolution + norm + cache write
 constexpr int CONV_MAX_TAPS = 16;
 constexpr int UNIT_MAX_PER_LANE = 8;        // a head is at most 64 * 8 = 512 channels wide
 
 struct ConvArgs {
   const void* x; long x_stride;             // [T, x_stride]: [q | k | v | ...]
-  const void* conv_w;                       // [C, taps]
+  const void* conv_w;                       // [taps, C] (tap-major: the taps of neighbouring channels side by side)
   void* state;                              // [slots, R, C], R = max(taps - 1, 1)
   const int* slots;                         // [B]
   const int* qsl;                           // [B + 1]
@@ -167,7 +249,7 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
           if (p >= chunk_start && p >= 0) uv = ldf(x + (long)(t - back) * a.x_stride + c);
           else if (p >= 0) uv = ldf(st + (long)(R - (chunk_start - p)) * C + c);
           hist[j] = uv;
-          v += ldf(w + (long)c * a.taps + j) * uv;
+          v += ldf(w + (long)j * C + c) * uv;
         }
         if (own_state) {
           for (int k = 0; k < R; ++k) stf(st + (long)k * C + c, hist[k + 1]);
@@ -268,9 +350,8 @@ __global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, in
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   if (live) {
-    // the taps of 8 channels are 8 * taps consecutive values
-    const T* wp = w + (long)c * a.taps;
     for (int j = 0; j < a.taps; ++j) {
+      const V8 wv = ld8<T>(w + (long)j * C + c);
       const int back = a.taps - 1 - j;
       const int p = pos - back;
       V8 u;
@@ -282,7 +363,7 @@ __global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, in
       }
       if (own_state && j >= 1) st8<T>(st + (long)(j - 1) * C + c, u);     // (row j - 1 was read one turn earlier)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)wp[e * a.taps + j] * (float)u[e];
+      for (int e = 0; e < 8; ++e) acc[e] += (float)wv[e] * (float)u[e];
     }
   }
   if (kind < 2) {
@@ -755,6 +836,14 @@ VDAMD_API int vdamd_scalar_norm_residual(void* out, const void* y, float* residu
   if (H <= 0 || (out != nullptr && g_next == nullptr)) return 1;
   const int th = norm_threads(H);
   int inner = 0;
+  if (y_dt != DT_F32 && y_dt == out_dt && H % 8 == 0 && y_stride % 8 == 0) {
+    return by_dtype(y_dt, [&](auto* ty) {
+      using TY = std::remove_pointer_t<decltype(ty)>;
+      if constexpr (!std::is_same_v<TY, float>)
+        hipLaunchKernelGGL((scalar_norm_residual_vec_kernel<TY>), dim3(rows), dim3(H >= 2048 ? 256 : 128), 0, stream,
+                           (TY*)out, (const TY*)y, residual, g_post, g_next, eps, H, y_stride);
+    });
+  }
   const int rc = by_dtype(y_dt, [&](auto* ty) {
     using TY = std::remove_pointer_t<decltype(ty)>;
     inner = by_dtype(out_dt, [&](auto* to) {
@@ -771,8 +860,16 @@ VDAMD_API int vdamd_poly_norm(void* out, const void* z, const float* coef, float
   if (rows <= 0) return 0;
   if (F <= 0) return 1;
   const int th = norm_threads(F);
+  const bool vec = dt != DT_F32 && F % 8 == 0 && z_stride % 8 == 0;
   return by_dtype(dt, [&](auto* tp) {
     using T = std::remove_pointer_t<decltype(tp)>;
+    if constexpr (!std::is_same_v<T, float>) {
+      if (vec) {
+        hipLaunchKernelGGL((poly_norm_vec_kernel<T>), dim3(rows), dim3(F >= 4096 ? 512 : 256), 0, stream, (T*)out,
+                           (const T*)z, coef, eps, F, z_stride);
+        return;
+      }
+    }
     hipLaunchKernelGGL((poly_norm_kernel<T>), dim3(rows), dim3(th), 0, stream, (T*)out, (const T*)z, coef, eps, F,
                        z_stride);
   });

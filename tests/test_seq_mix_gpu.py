@@ -58,7 +58,7 @@ def _conv_case(dtype, h, g, d, dv, taps, chunks, seed):
     b = len(chunks)
     n_rows = sum(n for _, n in chunks)
     x = torch.randn(n_rows, c + (8 if seed % 2 else h), device="cuda", generator=gen).to(dtype)
-    w = torch.randn(c, taps, device="cuda", generator=gen).to(dtype)
+    w = torch.randn(taps, c, device="cuda", generator=gen).to(dtype)
     state = torch.randn(b + 2, max(taps - 1, 1), c, device="cuda", generator=gen).to(dtype)
     slots = torch.randperm(b + 2, device="cuda", generator=gen)[:b].to(torch.int32)
     qsl = torch.tensor([0] + list(torch.tensor([n for _, n in chunks]).cumsum(0)), dtype=torch.int32, device="cuda")

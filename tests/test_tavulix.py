@@ -355,6 +355,7 @@ def test_short_convolution_carries_its_tail_across_portions(device, dtype, tol, 
     x = torch.randn(40, c, generator=gen).to(dt)
     w = torch.randn(c, taps, generator=gen).to(dt)
     want = oracle.causal_taps(x.double(), w.double())
+    w = w.t().contiguous()                                  # the op reads the taps tap-major
     state = torch.randn(3, max(taps - 1, 1), c, generator=gen).to(dt).to(device)        # stale tails
     ones = torch.ones(d, device=device)
     got, at = [], 0

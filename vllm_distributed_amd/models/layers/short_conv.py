@@ -29,6 +29,12 @@ class ShortConv(nn.Module):
         self.weight.weight_loader = self.load_piece          # type: ignore[attr-defined]
         self.state: Optional[torch.Tensor] = None
         self.dtype = dtype
+        # what the kernels read: the same numbers tap-major, ``[taps, channels]`` (the taps of neighbouring
+        # channels side by side: one 16-byte load per tap and lane); made once the checkpoint is in
+        self.register_buffer("weight_t", None)
+
+    def finalize_weights(self) -> None:
+        self.weight_t = self.weight.data.t().contiguous()
 
     def load_piece(self, param: nn.Parameter, w: torch.Tensor, shard_id: Optional[int] = None) -> None:
         from ..utils import materialize

@@ -69,7 +69,7 @@ class ConvAttentionMixer(nn.Module):
             return self.o(o), kept
         rows = None if md.num_prefills == 0 else md.token_rows(ctx.positions)[0]
         q, kept = ops.conv_norm_cache(
-            x, self.conv.weight, self.conv.state, md.state_slots, md.query_start_loc, md.seq_lens, rows, ctx.positions,
+            x, self.conv.weight_t, self.conv.state, md.state_slots, md.query_start_loc, md.seq_lens, rows, ctx.positions,
             self.heads, self.kv_heads, self.dim, self.vdim, self.q_norm, self.k_norm, self.eps,
             v_first, self.vmix if v_first is not None else None, provide_v,
             self.attn.k_cache, self.attn.v_cache, md.slot_mapping, md.num_prefills > 0)

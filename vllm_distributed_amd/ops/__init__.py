@@ -648,7 +648,7 @@ def poly_norm(z, coef, eps: float):
 def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
                     num_kv_heads: int, dim: int, vdim: int, q_norm, k_norm, eps: float, v_first, v_lambda,
                     keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
-    """Short convolution (with per-request state) + per-head q / k norm + value mixing + cache write over a fused
+    """``conv_weight`` is tap-major, ``[taps, C]``.  Short convolution (with per-request state) + per-head q / k norm + value mixing + cache write over a fused
     projection; see ``torch_ref.conv_norm_cache``.  ``token_seq`` (None: row ``t`` belongs to sequence ``t``) and
     ``positions`` tell the kernel which sequence and position each row has."""
     if _use_hip(x):

@@ -1286,11 +1286,11 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
                     keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
     t = x.shape[0]
     c = num_heads * dim + num_kv_heads * (dim + vdim)
-    taps = conv_weight.shape[1]
+    taps = conv_weight.shape[0]
     r = max(taps - 1, 1)
     b = seq_lens.shape[0]
     assert x.dim() == 2 and x.shape[1] >= c and x.stride(1) == 1 and x.is_cuda
-    assert conv_weight.shape == (c, taps) and conv_weight.dtype == x.dtype and conv_weight.is_contiguous()
+    assert conv_weight.shape == (taps, c) and conv_weight.dtype == x.dtype and conv_weight.is_contiguous()
     assert 1 <= taps <= CONV_MAX_TAPS and dim <= UNIT_MAX_WIDTH and vdim <= UNIT_MAX_WIDTH
     assert state is not None and state.dtype == x.dtype and state.is_contiguous() and state.shape[1:] == (r, c), \
         (None if state is None else state.shape, (r, c))

@@ -468,12 +468,12 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
 
 def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
                query_start_loc: torch.Tensor, seq_lens: torch.Tensor) -> torch.Tensor:
-    """Causal per-channel convolution over time of the packed rows ``x[T, C]`` with ``weight[C, taps]``:
-    ``y_t = sum_j weight[:, j] * u_(t - taps + 1 + j)``, zero before a sequence's first position.  Sequence ``i``
+    """Causal per-channel convolution over time of the packed rows ``x[T, C]`` with tap-major ``weight[taps, C]``:
+    ``y_t = sum_j weight[j] * u_(t - taps + 1 + j)``, zero before a sequence's first position.  Sequence ``i``
     owns rows ``query_start_loc[i]:query_start_loc[i+1]``, the last positions of its ``seq_lens[i]`` tokens; the
     ``taps - 1`` inputs in front of them come from ``state[slots[i]]`` (``[slots, taps - 1, C]``, oldest first),
     which is left holding the last ``taps - 1`` inputs of the sequence.  Returns fp32 ``[T, C]``."""
-    taps = weight.shape[1]
+    taps = weight.shape[0]
     r = taps - 1
     y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
     wf = weight.float()
@@ -491,7 +491,7 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, slots
         u = torch.cat([hist, x[s:e].float()], 0)
         acc = torch.zeros((n, x.shape[1]), dtype=torch.float32, device=x.device)
         for j in range(taps):
-            acc += wf[:, j] * u[j:j + n]
+            acc += wf[j] * u[j:j + n]
         y[s:e] = acc
         if r:
             state[sl[i]] = u[u.shape[0] - r:].to(state.dtype)
