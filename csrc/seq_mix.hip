@@ -315,15 +315,10 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
 // when that is a power of two (the per-head sum of squares is then a few xor-shuffles inside the lane group).
 // Wave tasks are numbered (token, task) across the grid: q and k units first, then v units.
 template <typename T>
-__global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, int gs_d, int upw_d, int gs_v, int upw_v,
-                                                                  int tasks_d, int tasks_v) {
+__device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int task, int gs_d, int upw_d, int gs_v,
+                                               int upw_v, int tasks_d) {
   using V8 = typename Vec8<T>::type;
   const int lane = threadIdx.x & 63;
-  const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const int tasks = tasks_d + tasks_v;
-  const int t = (int)(wid / tasks);
-  if (t >= a.T) return;
-  const int task = (int)(wid % tasks);
   const bool is_v = task >= tasks_d;
   const int gs = is_v ? gs_v : gs_d, upw = is_v ? upw_v : upw_d;
   const int sub = lane / gs;                      // unit within the wave
@@ -413,6 +408,21 @@ __global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, in
     T* dst = (T*)a.v_cache + (((blk * a.G + head) * (a.block_size >> 3) + (off >> 3)) * (long)width + 8 * li) * 8 + (off & 7);
 #pragma unroll
     for (int e = 0; e < 8; ++e) dst[e * 8] = (T)acc[e];
+  }
+}
+
+// A wave takes one task (a group of heads) of `tok_per_wave` consecutive rows: the index loads of the next row
+// overlap the arithmetic of the current one, and its taps are still in the cache.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, int gs_d, int upw_d, int gs_v, int upw_v,
+                                                                  int tasks_d, int tasks_v, int tok_per_wave) {
+  const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int tasks = tasks_d + tasks_v;
+  const long t0 = (wid / tasks) * tok_per_wave;
+  const int task = (int)(wid % tasks);
+  for (int i = 0; i < tok_per_wave; ++i) {
+    if (t0 + i >= a.T) return;                    // (the same for every lane of the wave)
+    conv_vec_token<T>(a, (int)(t0 + i), task, gs_d, upw_d, gs_v, upw_v, tasks_d);
   }
 }
 
@@ -903,9 +913,10 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
         pack(D, gs_d, upw_d);
         pack(Dv, gs_v, upw_v);
         const int tasks_d = (H + G + upw_d - 1) / upw_d, tasks_v = (G + upw_v - 1) / upw_v;
-        const long wtasks = (long)T * (tasks_d + tasks_v);
+        const int tok_per_wave = T >= 4096 ? 4 : (T >= 1024 ? 2 : 1);
+        const long wtasks = (long)((T + tok_per_wave - 1) / tok_per_wave) * (tasks_d + tasks_v);
         hipLaunchKernelGGL((conv_norm_cache_vec_kernel<TT>), dim3((unsigned)((wtasks + 3) / 4)), dim3(256), 0, stream, a,
-                           gs_d, upw_d, gs_v, upw_v, tasks_d, tasks_v);
+                           gs_d, upw_d, gs_v, upw_v, tasks_d, tasks_v, tok_per_wave);
       }
     }
     if (!vec || std::is_same_v<TT, float>)

@@ -50,11 +50,11 @@ def test_poly_norm(dtype, f):
     _close(hip.poly_norm(z, coef, 1e-5), torch_ref.poly_norm(z, coef, 1e-5), dtype, 8)
 
 
-def _conv_case(dtype, h, g, d, dv, taps, chunks, seed):
+def _conv_case(dtype, h, g, d, dv, taps, chunks, seed, nblocks=64):
     """Sequences given as (tokens already run, tokens in this step); rows in batch order."""
     gen = torch.Generator(device="cuda").manual_seed(seed)
     c = h * d + g * (d + dv)
-    bs, nblocks = 16, 64
+    bs = 16
     b = len(chunks)
     n_rows = sum(n for _, n in chunks)
     x = torch.randn(n_rows, c + (8 if seed % 2 else h), device="cuda", generator=gen).to(dtype)
@@ -200,3 +200,25 @@ def test_embed_positions(dtype, h):
     got = hip.embed_positions(ids, ps, emb, pos)
     assert got.dtype == torch.float32
     assert torch.equal(got, emb[ids.long()].float() + pos[ps.long()].float())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_conv_norm_cache_long_chunks(dtype):
+    """Thousands of rows in one launch (a wave then takes several consecutive rows), chunk borders inside a wave's
+    rows, a decode row and a two-row chunk between the long ones."""
+    hip = _hip()
+    h, g, d, dv, taps = 4, 2, 64, 32, 4
+    chunks = [(0, 2999), (5, 1501), (7, 1), (0, 2), (100, 700)]
+    c = _conv_case(dtype, h, g, d, dv, taps, chunks, seed=11, nblocks=5 * 200)
+    s1, s2 = c["state"].clone(), c["state"].clone()
+    k1, v1, k2, v2 = c["kc"].clone(), c["vc"].clone(), c["kc"].clone(), c["vc"].clone()
+    args = (h, g, d, dv, c["qn"], c["kn"], 1e-5, c["vf"], c["lam"], False)
+    q1, _ = hip.conv_norm_cache(c["x"], c["w"], s1, c["slots"], c["qsl"], c["seq_lens"], c["tok_seq"], c["pos"], *args,
+                                k1, v1, c["slot_map"], True)
+    q2, _ = torch_ref.conv_norm_cache(c["x"], c["w"], s2, c["slots"], c["qsl"], c["seq_lens"], *args, k2, v2, c["slot_map"])
+    _close(q1, q2, dtype, 4)
+    _close(k1, k2, dtype, 4)
+    _close(v1, v2, dtype, 8)
+    for i, (a, n) in enumerate(chunks):
+        first = max(0, (taps - 1) - (a + n))
+        _close(s1[int(c["slots"][i]), first:], s2[int(c["slots"][i]), first:], dtype, 1e-6)
