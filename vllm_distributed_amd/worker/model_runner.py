@@ -256,7 +256,7 @@ class ModelRunner:
         self.graph_pool = None
         self.graph_fallback_reason: Optional[str] = "not captured yet"
         self._static: Dict[str, torch.Tensor] = {}
-        self._stage_copied = None         # event behind the last step's copies out of the pinned staging tensors
+        self._stages: List[Dict[str, torch.Tensor]] = []      # pinned staging of the decode graphs' inputs (two sets)
         self.decode_workspace: Optional[torch.Tensor] = None
         self.draft = None                 # worker.draft_model.DraftProposer (draft-model speculation)
         # vision-language requests: their images (multimodal.MultiModalInput) and the projected features of
@@ -1190,8 +1190,12 @@ class ModelRunner:
         }
         if self.is_gpu:
             # pinned staging so one H2D per tensor per step
-            self._stage = {k: torch.zeros_like(v, device="cpu").pin_memory()
-                           for k, v in self._static.items() if k != "qsl"}
+            # two sets, used in turn: the device reads a set when the copies out of it run, which under async
+            # scheduling is up to a step after they were issued
+            self._stages = [{k: torch.zeros_like(v, device="cpu").pin_memory()
+                             for k, v in self._static.items() if k != "qsl"} for _ in range(2)]
+            self._stage_events = [None, None]
+            self._stage_turn = 0
 
     def _static_metadata(self, bs: int, max_seq_len: int) -> AttentionMetadata:
         s = self._static
@@ -1334,13 +1338,16 @@ class ModelRunner:
         return g
 
     def _run_graph(self, g: DecodeGraph, p: dict):
-        s, st = self._static, self._stage
+        turn = self._stage_turn % 2
+        self._stage_turn += 1
+        s, st = self._static, self._stages[turn]
         n, bs = len(p["req_ids"]), g.batch_size
         mb = p["max_blocks"]
         # the pinned staging tensors are read by the device when the copies below run, not when they are issued:
-        # a step that nobody waits for (nothing sampled, no logits asked) must not have them rewritten under it
-        if self._stage_copied is not None:
-            self._stage_copied.synchronize()
+        # a set is rewritten only once the copies of the replay before last, which used it, have run (no wait in
+        # practice; a step that nobody waits for - nothing sampled, no logits asked - is what makes it matter)
+        if self._stage_events[turn] is not None:
+            self._stage_events[turn].synchronize()
         st["input_ids"][:n] = torch.from_numpy(p["input_ids"])
         st["positions"][:n] = torch.from_numpy(p["positions"])
         st["slot_mapping"][:n] = torch.from_numpy(p["slot_mapping"])
@@ -1360,9 +1367,9 @@ class ModelRunner:
             s[k][:bs].copy_(st[k][:bs], non_blocking=True)
         s["block_table"][:n, :mb].copy_(st["block_table"][:n, :mb], non_blocking=True)
         self._patch_unknown_inputs(s["input_ids"], p)
-        if self._stage_copied is None:
-            self._stage_copied = torch.cuda.Event()
-        self._stage_copied.record()
+        if self._stage_events[turn] is None:
+            self._stage_events[turn] = torch.cuda.Event()
+        self._stage_events[turn].record()
         if self.pp_link is not None:
             # the stage's layers are the graph; the transfers around it run on the link's streams
             if not self.pp.is_first_rank:
