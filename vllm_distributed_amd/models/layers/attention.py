@@ -249,6 +249,12 @@ class WindowBiasAttention(Attention):
     def kv_values_per_token(self) -> int:
         return self.num_kv_heads * (self.head_dim + self.vdim)
 
+    def bind_kv_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_scales: Optional[tuple] = None) -> None:
+        if k_cache.dtype == torch.float8_e4m3fn:
+            raise ValueError("an e4m3 KV cache is not supported for attention over convolved, normalised keys "
+                             "(its kernels read the cache in the model dtype); use --kv-cache-dtype auto")
+        super().bind_kv_cache(k_cache, v_cache, kv_scales)
+
     def forward_cached(self, q: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``q[T, Hq, dim]`` (this step's keys and values already cached), ``gate[T, Hq]`` raw -> ``[T, Hq * vdim]``."""
         md = _CTX.attn_metadata
