@@ -321,8 +321,9 @@ __device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int tas
   const int lane = threadIdx.x & 63;
   const bool is_v = task >= tasks_d;
   const int gs = is_v ? gs_v : gs_d, upw = is_v ? upw_v : upw_d;
-  const int sub = lane / gs;                      // unit within the wave
-  const int li = lane % gs;                       // lane within the unit
+  // unit within the wave, lane within the unit (several units per wave only when gs is a power of two)
+  const int sub = upw > 1 ? lane >> __builtin_ctz(gs) : lane / gs;
+  const int li = upw > 1 ? lane & (gs - 1) : lane - sub * gs;
   const int unit = (is_v ? task - tasks_d : task) * upw + sub;
   const int n_units = is_v ? a.G : a.H + a.G;
   const bool live = sub < upw && unit < n_units;
@@ -398,7 +399,9 @@ __device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int tas
   }
   const int slot = a.slot_mapping[t];
   if (slot < 0 || a.k_cache == nullptr) return;
-  const long blk = slot / a.block_size, off = slot % a.block_size;
+  long blk, off;
+  if ((a.block_size & (a.block_size - 1)) == 0) { blk = slot >> __builtin_ctz(a.block_size); off = slot & (a.block_size - 1); }
+  else { blk = slot / a.block_size; off = slot % a.block_size; }
   if (kind == 1) {
     V8 o;
 #pragma unroll
@@ -416,10 +419,9 @@ __device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int tas
 template <typename T>
 __global__ __launch_bounds__(256) void conv_norm_cache_vec_kernel(ConvArgs a, int gs_d, int upw_d, int gs_v, int upw_v,
                                                                   int tasks_d, int tasks_v, int tok_per_wave) {
-  const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const int tasks = tasks_d + tasks_v;
-  const long t0 = (wid / tasks) * tok_per_wave;
-  const int task = (int)(wid % tasks);
+  // grid (row groups / 4, tasks): no division to find the wave's place
+  const long t0 = ((long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * tok_per_wave;
+  const int task = blockIdx.y;
   for (int i = 0; i < tok_per_wave; ++i) {
     if (t0 + i >= a.T) return;                    // (the same for every lane of the wave)
     conv_vec_token<T>(a, (int)(t0 + i), task, gs_d, upw_d, gs_v, upw_v, tasks_d);
@@ -657,6 +659,12 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   const T* kc = (const T*)a.k_cache;
   const T* vc = (const T*)a.v_cache;
   const int bs = a.block_size, bs8 = a.block_size >> 3;
+  // block sizes are powers of two in practice: key -> (block, offset) by shift and mask instead of two divisions
+  const int bs_shift = (bs & (bs - 1)) == 0 ? __builtin_ctz(bs) : -1;
+  auto split = [&](int key, int& bi, int& off) {
+    if (bs_shift >= 0) { bi = key >> bs_shift; off = key & (bs - 1); }
+    else { bi = key / bs; off = key - bi * bs; }
+  };
   f32x4 acc[VT];
 #pragma unroll
   for (int c = 0; c < VT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -676,9 +684,12 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     // K rows of the two interleaved tiles
     const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
     const int ka = min(key0, p_last), kb = min(key0 + 4, p_last);
-    const long blk_a = bt[ka / bs], blk_b = bt[kb / bs];
-    const T* kpa = kc + ((blk_a * a.G + g) * bs + (ka % bs)) * (long)D + 8 * g4;
-    const T* kpb = kc + ((blk_b * a.G + g) * bs + (kb % bs)) * (long)D + 8 * g4;
+    int bi_a, off_a, bi_b, off_b, bi_v, off_v;
+    split(ka, bi_a, off_a);
+    split(kb, bi_b, off_b);
+    const long blk_a = bt[bi_a], blk_b = bt[bi_b];
+    const T* kpa = kc + ((blk_a * a.G + g) * bs + off_a) * (long)D + 8 * g4;
+    const T* kpb = kc + ((blk_b * a.G + g) * bs + off_b) * (long)D + 8 * g4;
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < DT; ++k) {
@@ -687,8 +698,9 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     }
     // V^T rows: this lane's 8 keys are base + 8 * g4 .. + 7, channel 16 * c + r16
     const int vkey = min(base + 8 * g4, p_last) & ~7;
-    const long blk_v = bt[vkey / bs];
-    const T* vp = vc + (((blk_v * a.G + g) * bs8 + ((vkey % bs) >> 3)) * (long)DV + r16) * 8;
+    split(vkey, bi_v, off_v);
+    const long blk_v = bt[bi_v];
+    const T* vp = vc + (((blk_v * a.G + g) * bs8 + (off_v >> 3)) * (long)DV + r16) * 8;
     V8 vf[VT];
 #pragma unroll
     for (int c = 0; c < VT; ++c) vf[c] = ld8<T>(vp + (long)c * 128);
@@ -914,9 +926,9 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
         pack(Dv, gs_v, upw_v);
         const int tasks_d = (H + G + upw_d - 1) / upw_d, tasks_v = (G + upw_v - 1) / upw_v;
         const int tok_per_wave = T >= 4096 ? 4 : (T >= 1024 ? 2 : 1);
-        const long wtasks = (long)((T + tok_per_wave - 1) / tok_per_wave) * (tasks_d + tasks_v);
-        hipLaunchKernelGGL((conv_norm_cache_vec_kernel<TT>), dim3((unsigned)((wtasks + 3) / 4)), dim3(256), 0, stream, a,
-                           gs_d, upw_d, gs_v, upw_v, tasks_d, tasks_v, tok_per_wave);
+        const int groups = (T + tok_per_wave - 1) / tok_per_wave;
+        hipLaunchKernelGGL((conv_norm_cache_vec_kernel<TT>), dim3((groups + 3) / 4, tasks_d + tasks_v), dim3(256), 0,
+                           stream, a, gs_d, upw_d, gs_v, upw_v, tasks_d, tasks_v, tok_per_wave);
       }
     }
     if (!vec || std::is_same_v<TT, float>)
