@@ -79,7 +79,7 @@ def _conv_case(dtype, h, g, d, dv, taps, chunks, seed, nblocks=64):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(4, 2, 32, 16, 3), (6, 3, 64, 48, 4), (2, 1, 24, 8, 2), (3, 3, 128, 128, 1),
-                                   (2, 2, 72, 40, 5)])
+                                   (2, 2, 72, 40, 5), (2, 1, 20, 12, 3), (3, 1, 7, 5, 9)])
 @pytest.mark.parametrize("mix", [False, True])
 def test_conv_norm_cache(dtype, shape, mix):
     hip = _hip()
@@ -125,7 +125,7 @@ def test_conv_decode_rows_own_their_state():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(12, 3, 64, 32), (6, 3, 32, 48), (4, 1, 16, 16), (4, 4, 128, 128), (2, 2, 72, 8),
-                                   (40, 2, 64, 64)])
+                                   (40, 2, 64, 64), (2, 2, 20, 12), (3, 1, 7, 5)])
 @pytest.mark.parametrize("window,keep", [(0, 0), (20, 0), (20, 3), (200, 7), (1, 2), (40, 70)])
 @pytest.mark.parametrize("mfma", [True, False])
 def test_window_bias_attention(dtype, shape, window, keep, mfma, monkeypatch):
