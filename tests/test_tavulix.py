@@ -258,6 +258,48 @@ def test_batch_rows_equal_single_runs(device, dtype, tol, tmp_path_factory, tmp_
         assert d <= (1e-4 if dtype == "float32" else 0.2), (p, float(d))
 
 
+@pytest.mark.parametrize("device,dtype,tol", DEVICES)
+def test_pages_behind_the_window_are_reused_while_the_request_goes_on(device, dtype, tol, tmp_path_factory, tmp_path):
+    """A long request leaves its window behind: the pages over the keys no layer sees any more go back to the pool
+    (those over the kept first keys stay), short requests that come and go take them, and the long request's own
+    later pages come from the same pool.  Its logits, and theirs, stay those of each request alone."""
+    from vllm_distributed_amd.entrypoints import trace_replay
+    path, cfg, w = model_dir("varied", tmp_path_factory)              # windows 9 / 5 / 17 / 3, kept 2 / 0 / 3 / 1
+    long_req, short = tokens_for(cfg, 420, 30), tokens_for(cfg, 40, 31)
+    reqs = {"long": long_req}
+    steps, at, k = [[("long", long_req[:250], [249])]], 250, 0
+    while at < len(long_req):
+        step = [("long", long_req[at:at + 1], [0])]
+        at += 1
+        ended = []
+        if at % 20 == 0 and k < 8:
+            k += 1
+            reqs[f"s{k}"] = short
+            step.append((f"s{k}", short, [len(short) - 1, 7]))
+            ended.append(f"s{k}")
+        if at == len(long_req):
+            ended.append("long")
+        steps.append(step + ([{"end": ended}] if ended else []))
+    released = []
+    original = trace_replay.replay
+
+    def spy(core, lines, out_dir, say=print):
+        kv = core.scheduler.kv
+        real = kv.release_out_of_window
+        kv.release_out_of_window = lambda r: released.append(real(r)) or released[-1]
+        return original(core, lines, out_dir, say)
+
+    trace_replay.replay = spy
+    try:
+        # 27 pages of 16 hold the long request alone; a short one beside it lives on pages the window has left
+        got = run_schedule(path, steps, dtype, device, max_tokens=448 + 64, tmp=tmp_path)
+    finally:
+        trace_replay.replay = original
+    assert sum(released) > 5
+    assert len(got) == 1 + 170 + 16
+    check(got, "varied", cfg, w, reqs, tol)
+
+
 # --------------------------------------------------------------------------- mechanisms alone, made to show
 def _attention_case(device, dtype, n, d, dv, bs=16):
     """One sequence of ``n`` keys in shuffled pages; the keys are orthogonal directions so that a query can single
