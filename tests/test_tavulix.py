@@ -484,6 +484,29 @@ def test_forced_steps_use_the_pools_and_refuse_what_does_not_fit(tmp_path_factor
         core.shutdown()
 
 
+def test_the_trace_runner_as_a_program(tmp_path_factory, tmp_path):
+    """``bin/trace_run`` itself: steps on standard input, one ``done <step>`` per step (also where nothing is
+    wanted), logits files only for steps that want some, exit code 0 at the end of the input."""
+    import subprocess
+    import sys
+    path, cfg, w = model_dir("degenerate", tmp_path_factory)
+    a, b = tokens_for(cfg, 9, 50), tokens_for(cfg, 5, 51)
+    lines = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]}, {"id": "b", "tokens": b[:2], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[2:], "want": []}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[6:], "want": [2]}], "end": ["a"]}]
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "trace_run")
+    r = subprocess.run([sys.executable, exe, "--model", path, "--dtype", "float32", "--out", str(tmp_path), "--max-tokens", "128",
+                        "--device", "cpu"], input="".join(json.dumps(x) + "\n" for x in lines), text=True,
+                       capture_output=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert sorted(f for f in os.listdir(tmp_path) if f.endswith(".f32")) == ["0.f32", "2.f32"]
+    want = oracle_logits("degenerate", cfg, w, a)
+    got0 = np.fromfile(tmp_path / "0.f32", dtype="<f4").reshape(2, cfg["vocab"])
+    got2 = np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(1, cfg["vocab"])
+    assert np.abs(got0 - want[[0, 5]]).max() < 2e-4 and np.abs(got2 - want[[8]]).max() < 2e-4
+
+
 # ------------------------------------------------------------------------------------------- generation
 @pytest.mark.parametrize("device,dtype", [pytest.param("cpu", "float32", id="cpu-f32"),
                                           pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
