@@ -126,6 +126,19 @@ def normalize_hf_config(cfg: Dict[str, Any]) -> None:
                      ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
             if cfg.get(k) is None and v is not None:
                 cfg[k] = v
+    if cfg.get("architecture") == "Kabapel" or cfg.get("model_type") == "kabapel":
+        # Kabapel lists its layers one by one as well; it has no position table, so nothing but the cache bounds a
+        # sequence (``max_positions`` is honoured when a config states one)
+        cfg.setdefault("model_type", "kabapel")
+        cfg.setdefault("architectures", ["KabapelForCausalLM"])
+        mixers = [l.get("mixer") or {} for l in cfg.get("layers") or []]
+        first = mixers[0] if mixers else {}
+        for k, v in (("hidden_size", cfg.get("width")), ("vocab_size", cfg.get("vocab")),
+                     ("max_position_embeddings", cfg.get("max_positions") or 131072), ("num_hidden_layers", len(mixers)),
+                     ("num_attention_heads", first.get("heads", 1)), ("num_key_value_heads", first.get("heads", 1)),
+                     ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
+            if cfg.get(k) is None and v is not None:
+                cfg[k] = v
     if cfg.get("model_type") == "dbrx":
         # DBRX nests its attention and expert settings
         a, f = cfg.get("attn_config") or {}, cfg.get("ffn_config") or {}

@@ -124,7 +124,7 @@ class EngineCore:
             num_blocks = int(cc.num_gpu_blocks_override)
         else:
             seqs = self.vllm_config.scheduler_config.max_num_seqs       # (per-request layer state comes off the top)
-            num_blocks = min(int(max(a - seqs * getattr(s, "state_bytes_per_request", 0), 0) // s.bytes_per_block)
+            num_blocks = min(int(max(a - seqs * getattr(s, "state_bytes_per_request", 0), 0) // max(s.bytes_per_block, 1))
                              for a, s in zip(avail, specs))
             # no point holding more than every sequence at full length
             cap = self.vllm_config.scheduler_config.max_num_seqs * cdiv(

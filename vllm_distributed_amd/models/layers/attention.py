@@ -218,6 +218,81 @@ class LatentAttention(Attention):
         return ops.mla_attention(q, self.k_cache, self.v_cache, md.block_table, rows, lens, self.scale, md.max_seq_len)
 
 
+def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
+    """Angular frequencies of a rotation over ``dims`` values paired half-apart, ``f_i = base^(-2i / dims)`` for
+    ``i < dims / 2``, as an fp32 tensor, and the factor both cos and sin are multiplied by.  ``scaling`` =
+    ``{factor, original, fast, slow}`` blends towards ``f_i / factor`` the YaRN way: with ``d(r) = dims *
+    ln(original / (2 pi r)) / (2 ln base)`` the index at which a pair turns ``r`` times within ``original``
+    positions, a ramp rises linearly from 0 at ``max(floor(d(fast)), 0)`` to 1 at ``min(ceil(d(slow)), dims - 1)``;
+    pair ``i`` gets ``ramp_i f_i / factor + (1 - ramp_i) f_i``, and the factor is ``0.1 ln(factor) + 1``."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    scale = 1.0
+    if scaling:
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+
+        def index_of(turns: float) -> float:
+            return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+        lo = max(math.floor(index_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(index_of(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        scale = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32), float(scale)
+
+
+class RowLatentAttention(Attention):
+    """Latent attention over ONE row cache: a token's row is ``[normalised latent (rank) | rotated shared key part
+    (rope)]``, its first ``rank`` values are also its value, and the per-head up-projections are folded into the
+    query and the output by the caller.  Any ``rank`` / ``rope``; the rotation is computed from ``inv_freq`` in the
+    kernel (positions and angles in fp32), so no table bounds the positions; scores, softmax and the weighted sum are
+    fp32 in every dtype.  ``source``: another layer's instance whose rows this layer reads instead of keeping its own
+    (layers that share keys and values: the reader allocates nothing and writes nothing)."""
+    latent = True
+    row_cache = True
+
+    def __init__(self, num_heads: int, rank: int, rope: int, scale: float, layer_idx: int,
+                 source: Optional["RowLatentAttention"] = None):
+        super().__init__(num_heads, rank + rope, 1, scale, layer_idx)
+        self.rank, self.rope, self.v_dim = rank, rope, rank
+        if source is not None and (source.rank, source.rope) != (rank, rope):
+            raise ValueError(f"layer {layer_idx} reads the latent rows of layer {source.layer_idx}, which have "
+                             f"another shape ({source.rank} + {source.rope} against {rank} + {rope})")
+        # (kept out of the module tree: the owner is registered where it lives)
+        object.__setattr__(self, "source", source)
+
+    def kv_cache_shapes(self, num_blocks: int, block_size: int):
+        return (num_blocks, 1, block_size, self.head_dim), (num_blocks, 0)
+
+    def kv_values_per_token(self) -> int:
+        return self.head_dim
+
+    def bind_kv_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_scales: Optional[tuple] = None) -> None:
+        if k_cache.dtype == torch.float8_e4m3fn:
+            raise ValueError("an e4m3 KV cache is not supported for latent rows read in the model dtype; "
+                             "use --kv-cache-dtype auto")
+        super().bind_kv_cache(k_cache, v_cache, kv_scales)
+
+    @property
+    def rows(self) -> Optional[torch.Tensor]:
+        return (self.source if self.source is not None else self).k_cache
+
+    def forward_latent(self, q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
+                       norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor,
+                       rot_scale: float) -> torch.Tensor:
+        """``q[T, H, nope + rope]``, ``q_lat[H, T, rank]``, ``latent[T, rank + rope]`` (None for a reader of another
+        layer's rows): norm, rotations, cache write and query assembly in one op, then attention -> ``[T, H, rank]``."""
+        md, pos = _CTX.attn_metadata, _CTX.positions
+        write = latent is not None and self.source is None and md is not None
+        qf = ops.latent_prep(q, nope, q_lat, latent if write else None, norm_weight, eps, inv_freq, rot_scale, pos,
+                             self.k_cache if write else None, md.slot_mapping if write else None)
+        if md is None:                          # memory-profiling pass: no cache bound
+            return qf[..., :self.rank].contiguous()
+        rows, lens = md.token_rows(pos)
+        return ops.latent_row_attention(qf, self.rows, md.block_table, rows, lens, self.scale, self.rank, md.max_seq_len)
+
+
 class WindowBiasAttention(Attention):
     """Attention whose window keeps the first keys of the sequence, with a logarithmic distance bias instead of
     a rotation, an optional score cap, a sink in the softmax denominator and a sigmoid gate on each head's output;
@@ -323,3 +398,21 @@ class LayerNorm(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.layer_norm(x, self.weight, self.bias, self.eps)
+
+
+class ResidualLayerNorm(nn.Module):
+    """Layer norm with weight and bias over an fp32 residual stream, in fp32 arithmetic (parameters kept in fp32);
+    ``forward`` returns the model dtype (the input of a projection), ``add`` folds a sublayer's output into the
+    stream and hands back the normed sum in the same launch."""
+
+    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, bias: bool = True):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=torch.float32), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=torch.float32), requires_grad=False) if bias else None
+        self.eps, self.dtype = eps, dtype
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.layer_norm_to(x, self.weight, self.bias, self.eps, out_dtype or self.dtype)
+
+    def add(self, y: torch.Tensor, residual: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.add_layer_norm(y, residual, self.weight, self.bias, self.eps, out_dtype or self.dtype)

@@ -348,3 +348,161 @@ class FusedMoE(nn.Module):
         if reduce and self.tp > 1:
             out = tensor_model_parallel_all_reduce(out)
         return out
+
+
+def _ceil128(n: int) -> int:
+    return (n + 127) // 128 * 128
+
+
+class ClampedGluMLP(nn.Module):
+    """One feed-forward of the clamped GLU form, ``down(g sigmoid(alpha g) (u + 1))`` with ``g = min(gate(x),
+    limit)`` and ``u = clamp(up(x), -limit, limit)``, gate and up as one fused projection; no biases."""
+
+    def __init__(self, hidden: int, inter: int, limit: float, alpha: float, dtype: torch.dtype):
+        super().__init__()
+        self.inter, self.limit, self.alpha = inter, float(limit), float(alpha)
+        self.w13 = nn.Parameter(torch.empty(2 * inter, hidden, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.empty(hidden, inter, dtype=dtype), requires_grad=False)
+        self.w13.weight_loader = self._load_w13
+
+    def _load_w13(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        param.data.narrow(0, int(shard_id) * self.inter, self.inter).copy_(materialize(w))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.linear(ops.clamped_glu(ops.linear(x, self.w13), self.limit, self.alpha), self.w2)
+
+
+class GroupedIdentityMoE(FusedMoE):
+    """Routed experts of the clamped GLU form behind a softmax router with a per-output correction that only steers
+    the choice, expert groups of neighbours (a group scores as its best member; only the best ``keep_groups`` groups
+    stay eligible, the others count as minus infinity), renormalised weights, and ``identity`` trailing router
+    outputs that stand for experts whose output is their input; plus an optional always-on shared expert scaled by
+    ``sigmoid(shared_gate . x)``, one number per token.
+
+    The router is fp32 (weights and product); the choice is made on ``softmax + correction``, the weights are the
+    chosen outputs' softmax values over their sum.  On the GPU in 16-bit types the experts run as two grouped GEMMs
+    over expert-sorted rows with their reduction dimensions zero-padded to the kernels' 128-deep tiles: the identity
+    outputs are routed like experts held by nobody (no rows, no weights) and their share ``x * sum of their weights``
+    is added at the end.  Elsewhere (fp32, CPU) the experts run one after the other on the library GEMM."""
+    custom_routing = True
+
+    def __init__(self, hidden: int, inter: int, num_experts: int, identity: int, top_k: int, limit: float,
+                 dtype: torch.dtype, groups: int = 1, keep_groups: int = 1, alpha: float = 1.702,
+                 shared_inter: int = 0, shared_limit: Optional[float] = None):
+        outputs = num_experts + identity
+        super().__init__(hidden, inter, outputs, top_k, True, dtype, expert_parallel=False, allocate_experts=False)
+        if self.tp > 1:
+            raise NotImplementedError("GroupedIdentityMoE runs unsharded")
+        if groups < 1 or outputs % groups or not 1 <= keep_groups <= groups:
+            raise ValueError(f"{outputs} router outputs do not form {groups} equal groups of which {keep_groups} are kept")
+        if top_k > outputs:
+            raise ValueError(f"top {top_k} of {outputs} router outputs")
+        self.quant = None
+        self.real_experts, self.identity = num_experts, identity
+        self.local_experts, self.expert_start = num_experts, 0      # the identity outputs have no weights
+        self.groups, self.keep_groups = groups, keep_groups
+        self.limit, self.alpha = float(limit), float(alpha)
+        f32 = torch.float32
+        self.gate = ReplicatedLinear(hidden, outputs, False, f32, quant=False)
+        self.gate.e_score_correction_bias = nn.Parameter(torch.zeros(outputs, dtype=f32), requires_grad=False)
+        self.h_pad, self.i_pad = _ceil128(hidden), _ceil128(inter)
+        E = num_experts
+        # [gate rows ; up rows] (each padded to i_pad rows) x (reduction padded to h_pad); [hidden, i_pad]
+        self.w13 = nn.Parameter(torch.zeros(E, 2 * self.i_pad, self.h_pad, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.zeros(E, hidden, self.i_pad, dtype=dtype), requires_grad=False)
+        self.w13.weight_loader = self._load_w13
+        self.w2.weight_loader = self._load_w2
+        self.shared = ClampedGluMLP(hidden, shared_inter, self.limit if shared_limit is None else shared_limit,
+                                    alpha, dtype) if shared_inter else None
+        self.shared_gate = ReplicatedLinear(hidden, 1, False, dtype, quant=False) if shared_inter else None
+
+    # ------------------------------------------------------------------ loading
+    def _load_w13(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        e, which = shard_id                  # which: 0 = gate, 1 = up
+        dst = param.data[e, which * self.i_pad:(which + 1) * self.i_pad]
+        dst.zero_()                          # (the padding included: the loader poisons fresh parameters)
+        dst[:self.inter, :self.hidden].copy_(materialize(w))
+
+    def _load_w2(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        e, _ = shard_id
+        param.data[e].zero_()
+        param.data[e, :, :self.inter].copy_(materialize(w))
+
+    # ------------------------------------------------------------------ routing
+    def router_logits(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x.float(), self.gate.weight)
+
+    def route(self, logits: torch.Tensor):
+        scores = torch.softmax(logits.float(), dim=-1)
+        choice = scores + self.gate.e_score_correction_bias
+        if self.groups > 1 and self.keep_groups < self.groups:
+            per_group = choice.view(-1, self.groups, self.num_experts // self.groups).amax(-1)
+            best = per_group.topk(self.keep_groups, dim=-1).indices
+            keep = torch.zeros_like(per_group, dtype=torch.bool).scatter_(1, best, True)
+            keep = keep.unsqueeze(-1).expand(-1, self.groups, self.num_experts // self.groups).reshape(choice.shape)
+            choice = choice.masked_fill(~keep, float("-inf"))
+        topi = choice.topk(self.top_k, dim=-1).indices
+        topw = scores.gather(1, topi)
+        return topw / (topw.sum(-1, keepdim=True) + 1e-20), topi
+
+    # ------------------------------------------------------------------ compute
+    def _pad(self, x: torch.Tensor) -> torch.Tensor:
+        return x if self.h_pad == self.hidden else F.pad(x, (0, self.h_pad - self.hidden))
+
+    def _expert_mlp(self, e: int, x: torch.Tensor) -> torch.Tensor:
+        h = F.linear(self._pad(x), self.w13[e])
+        return F.linear(ops.clamped_glu(h, self.limit, self.alpha), self.w2[e])
+
+    def _grouped_tile_rows(self, x: torch.Tensor) -> int:
+        if self.num_experts > 512 or self.top_k > 16 or self.groups > 64 or x.dim() != 2 or self.hidden % 8:
+            return 0
+        return super()._grouped_tile_rows(x)
+
+    def _identity_share(self, topw: torch.Tensor, topi: torch.Tensor) -> Optional[torch.Tensor]:
+        if not self.identity:
+            return None
+        return (topw * (topi >= self.real_experts)).sum(-1, keepdim=True)
+
+    def decode_capturable(self, dtype: torch.dtype) -> bool:
+        """Whether a decode step of this block runs without a host synchronisation (the grouped path)."""
+        return dtype in (torch.bfloat16, torch.float16) and self.hidden % 8 == 0 and self.num_experts <= 512
+
+    def _forward_routed(self, x: torch.Tensor) -> torch.Tensor:
+        logits = self.router_logits(x)
+        tile_rows = self._grouped_tile_rows(x)
+        if tile_rows:
+            grouped = self.groups if self.keep_groups < self.groups else 1
+            topw, topi = ops.moe_topk_grouped(logits, self.gate.e_score_correction_bias, self.top_k, grouped,
+                                              self.keep_groups if grouped > 1 else 1, False, False, True, 1.0)
+            src_row, inv, tiles = ops.moe_align_fused(topi, self.num_experts, tile_rows, 0, self.real_experts)
+            xs = self._pad(x).index_select(0, src_row)
+            h = ops.grouped_linear(xs, tiles, tile_rows, weight=self.w13)
+            y = ops.grouped_linear(ops.clamped_glu(h, self.limit, self.alpha), tiles, tile_rows, weight=self.w2)
+            out = ops.moe_combine(y, topw, topi, inv, 0, self.real_experts)
+            share = self._identity_share(topw, topi.long())
+            return out if share is None else out + (x.float() * share).to(x.dtype)
+        topw, topi = self.route(logits)
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        flat_e = topi.reshape(-1)
+        order = flat_e.argsort(stable=True)
+        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()
+        tok = order // self.top_k
+        wts = topw.reshape(-1)[order]
+        start = 0
+        for eid, n in enumerate(counts[:self.real_experts]):
+            if n:
+                seg = slice(start, start + n)
+                rows = tok[seg]
+                out.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
+            start += n
+        share = self._identity_share(topw, topi)
+        if share is not None:
+            out += x.float() * share
+        return out.to(x.dtype)
+
+    def forward(self, x: torch.Tensor, reduce: bool = True, staged: bool = False, deferred: bool = False):
+        out = self._forward_routed(x)
+        if self.shared is not None:
+            g = torch.sigmoid(self.shared_gate(x).float())
+            out = (out.float() + self.shared(x).float() * g).to(x.dtype)
+        return out

@@ -51,6 +51,9 @@ def _weight_shapes(c: dict, arch: str) -> Dict[str, Tuple[int, ...]]:
     if arch in ("TavulixForCausalLM", "Tavulix"):
         from .tavulix import weight_shapes
         return weight_shapes(c)
+    if arch in ("KabapelForCausalLM", "Kabapel"):
+        from .kabapel import weight_shapes
+        return weight_shapes(c)
     if arch == "MedusaModel":
         h = c["hidden_size"]
         out = {}
@@ -454,6 +457,10 @@ def dummy_weights_iterator(mc: ModelConfig, device: torch.device,
         gen.manual_seed(_seed_for(name, mc.seed))
         if mc.architecture in ("TavulixForCausalLM", "Tavulix"):
             from .tavulix import random_weight
+            yield name, random_weight(name, shape, gen, device, dtype)
+            continue
+        if mc.architecture in ("KabapelForCausalLM", "Kabapel"):
+            from .kabapel import random_weight
             yield name, random_weight(name, shape, gen, device, dtype)
             continue
         if awq and _QUANTIZED_LINEAR.search(name) and shape[1] % g == 0 and shape[0] % 8 == 0:

@@ -67,6 +67,10 @@ _MODELS: Dict[str, Tuple[str, str]] = {
     # learned positions, convolved q / k / v, windowed attention with kept first keys, PolyNorm feed-forward
     "TavulixForCausalLM": ("tavulix", "TavulixForCausalLM"),
     "Tavulix": ("tavulix", "TavulixForCausalLM"),
+    # fp32 residual stream; decayed linear attention with a state per request beside latent attention over shared
+    # rows; grouped routing with identity experts
+    "KabapelForCausalLM": ("kabapel", "KabapelForCausalLM"),
+    "Kabapel": ("kabapel", "KabapelForCausalLM"),
     # draft heads of speculative decoding (never a served model by themselves; worker/draft_model.py)
     "EagleLlamaForCausalLM": ("spec_heads", "EagleLlamaForCausalLM"),
     "Eagle3LlamaForCausalLM": ("spec_heads", "Eagle3LlamaForCausalLM"),
@@ -78,7 +82,7 @@ _MODELS: Dict[str, Tuple[str, str]] = {
 
 # architectures whose layers keep per-request state besides the KV cache (convolution tails, recurrences): a cached
 # prefix's blocks do not bring that state back, so prefix reuse is off for them
-_KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix"}
+_KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix", "KabapelForCausalLM", "Kabapel"}
 
 
 def keeps_request_state(arch: str) -> bool:

@@ -676,3 +676,71 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         out.copy_(res)
         return out
     return res
+
+
+# ------------------------------------------------ fp32 residual stream with layer norms, decayed linear attention,
+# ------------------------------------------------ gated norm, clamped GLU, latent attention over one row cache
+def embed_scaled(ids, weight, scale: float):
+    """``weight[ids] * scale`` as the fp32 residual stream."""
+    if _use_hip(weight):
+        return _hip.embed_scaled(ids, weight, scale)
+    return torch_ref.embed_scaled(ids, weight, scale)
+
+
+def layer_norm_to(x, weight, bias, eps: float, out_dtype):
+    """Layer norm in fp32 arithmetic of rows of any float type, result in ``out_dtype``."""
+    if _use_hip(x):
+        return _hip.layer_norm_to(x, weight, bias, eps, out_dtype)
+    return torch_ref.layer_norm_to(x, weight, bias, eps, out_dtype)
+
+
+def add_layer_norm(y, residual, weight, bias, eps: float, out_dtype):
+    """``residual += y`` on the fp32 residual stream and the layer norm of the sum in ``out_dtype``: one launch."""
+    if _use_hip(y):
+        return _hip.add_layer_norm(y, residual, weight, bias, eps, out_dtype)
+    return torch_ref.add_layer_norm(y, residual, weight, bias, eps, out_dtype)
+
+
+def decay_linear_attention(x, num_heads: int, dim: int, vdim: int, decay, state, slots, query_start_loc, seq_lens,
+                           silu: bool = True, max_query_len: int = 0, token_seq=None):
+    """Linear attention with a per-head decay and a per-request fp32 state; see
+    ``torch_ref.decay_linear_attention``.  ``max_query_len`` (0: unknown) and ``token_seq`` (the sequence of every
+    row, None: row ``t`` is sequence ``t``) only help the kernels choose their launch."""
+    if _use_hip(x):
+        return _hip.decay_linear_attention(x, num_heads, dim, vdim, decay, state, slots, query_start_loc, seq_lens,
+                                           silu, max_query_len)
+    return torch_ref.decay_linear_attention(x, num_heads, dim, vdim, decay, state, slots, query_start_loc, seq_lens, silu)
+
+
+def gated_rms_norm(o, weight, gate, eps: float, out_dtype):
+    if _use_hip(o):
+        return _hip.gated_rms_norm(o, weight, gate, eps, out_dtype)
+    return torch_ref.gated_rms_norm(o, weight, gate, eps, out_dtype)
+
+
+def clamped_glu(h, limit: float, alpha: float):
+    if _use_hip(h):
+        return _hip.clamped_glu(h, limit, alpha)
+    return torch_ref.clamped_glu(h, limit, alpha)
+
+
+def relu_squared(x):
+    if _use_hip(x):
+        return _hip.relu_squared(x)
+    return torch.relu(x).square_()
+
+
+def latent_prep(q, nope: int, q_lat, latent, norm_weight, eps: float, inv_freq, rot_scale: float, positions, cache,
+                slot_mapping):
+    if _use_hip(q):
+        return _hip.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
+                                slot_mapping)
+    return torch_ref.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
+                                 slot_mapping)
+
+
+def latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale: float, rank: int, max_seq_len: int = 0):
+    if _use_hip(q):
+        attention_calls["hip"] += 1
+        return _hip.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank, max_seq_len)
+    return torch_ref.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank)

@@ -581,3 +581,137 @@ def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     if gate is not None:
         out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
     return out.to(q.dtype)
+
+
+# ------------------------------------------------ fp32 residual stream with layer norms, decayed linear attention,
+# ------------------------------------------------ gated norm, clamped GLU, latent attention over one row cache
+def embed_scaled(ids: torch.Tensor, weight: torch.Tensor, scale: float) -> torch.Tensor:
+    """``weight[ids] * scale`` as the fp32 residual stream."""
+    return weight[ids.long()].float() * scale
+
+
+def layer_norm_to(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """Layer norm (mean taken off, biased variance, weight and bias) in fp32 arithmetic, result in ``out_dtype``."""
+    xf = x.float()
+    d = xf - xf.mean(-1, keepdim=True)
+    y = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    if bias is not None:
+        y = y + bias.float()
+    return y.to(out_dtype)
+
+
+def add_layer_norm(y: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                   eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``residual += y`` in place on the fp32 residual stream, then ``layer_norm_to`` of the sum."""
+    residual.add_(y.float())
+    return layer_norm_to(residual, weight, bias, eps, out_dtype)
+
+
+def decay_linear_attention(x: torch.Tensor, num_heads: int, dim: int, vdim: int, decay: torch.Tensor,
+                           state: torch.Tensor, slots: torch.Tensor, query_start_loc: torch.Tensor,
+                           seq_lens: torch.Tensor, silu: bool = True) -> torch.Tensor:
+    """Linear attention with one decay per head over the packed rows ``x[T, C]`` whose leading columns are
+    ``[q (H * dim) | k (H * dim) | v (H * vdim)]`` (``silu``: each passed through SiLU first).  Per head
+    ``S_t = decay[h] S_(t-1) + k_t v_t^T`` and ``o_t = S_t^T q_t``; ``S`` is ``state[slots[i]]`` (``[slots, H, dim,
+    vdim]`` fp32) for sequence ``i``, taken as zero when the rows start at position 0 whatever the slot held, and left
+    holding the state after the sequence's last row.  fp32 arithmetic; returns fp32 ``[T, H * vdim]``."""
+    t = x.shape[0]
+    h = num_heads
+    qs, vs = h * dim, h * vdim
+    xf = x[:, :2 * qs + vs].float()
+    if silu:
+        xf = F.silu(xf)
+    q = xf[:, :qs].reshape(t, h, dim)
+    k = xf[:, qs:2 * qs].reshape(t, h, dim)
+    v = xf[:, 2 * qs:].reshape(t, h, vdim)
+    out = torch.zeros((t, h, vdim), dtype=torch.float32, device=x.device)
+    d = decay.float().view(h, 1, 1)
+    qsl, sls, sl = query_start_loc.tolist(), seq_lens.tolist(), slots.tolist()
+    for i, n_ctx in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        if e == s:
+            continue
+        st = state[sl[i]].float().clone() if n_ctx - (e - s) > 0 else torch.zeros_like(state[sl[i]], dtype=torch.float32)
+        for r in range(s, e):
+            st = d * st + k[r].unsqueeze(2) * v[r].unsqueeze(1)
+            out[r] = torch.einsum("hkv,hk->hv", st, q[r])
+        state[sl[i]] = st.to(state.dtype)
+    return out.reshape(t, vs)
+
+
+def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """``o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate)`` over whole rows, fp32 arithmetic."""
+    of = o.float()
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def clamped_glu(h: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """``g sigmoid(alpha g) (u + 1)`` for ``h = [gate | up]`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit,
+    limit)``; fp32 arithmetic, result in ``h``'s dtype."""
+    f = h.shape[-1] // 2
+    g = h[..., :f].float().clamp(max=limit)
+    u = h[..., f:].float().clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(h.dtype)
+
+
+def rotate_half_first(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rot_scale: float) -> torch.Tensor:
+    """Rotate the first ``2 * len(inv_freq)`` values of the last dimension of fp32 ``x[T, ..., n]``, value ``i``
+    paired with value ``i + len(inv_freq)``, by the angle ``positions[t] * inv_freq[i]`` (fp32), cos and sin both
+    times ``rot_scale``; the rest passes unchanged."""
+    half = inv_freq.numel()
+    a = positions.float().view(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    cos, sin = torch.cos(a) * rot_scale, torch.sin(a) * rot_scale
+    u, v = x[..., :half], x[..., half:2 * half]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., 2 * half:]], dim=-1)
+
+
+def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
+                norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
+                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> torch.Tensor:
+    """Between the projections and the attention of a layer whose keys and values are one shared latent row per
+    token.  ``q[T, H, nope + rope]``, ``q_lat[H, T, rank]`` (the unrotated query part already multiplied into the
+    latent space): returns ``[T, H, rank + rope] = [q_lat | rotated q[..., nope:]]``.  With ``latent[T, rank + rope]``
+    the row ``[RMS norm of the first rank values * norm_weight | rotated last rope values]`` goes into
+    ``cache[blocks, 1, block, rank + rope]`` at ``slot_mapping`` (a layer that reads another layer's rows passes
+    None).  Norm and rotation in fp32."""
+    t = q.shape[0]
+    q_rot = rotate_half_first(q[..., nope:].float(), positions[:t], inv_freq, rot_scale)
+    out = torch.cat([q_lat.transpose(0, 1).float(), q_rot], dim=-1).to(q.dtype)
+    if latent is not None and cache is not None and slot_mapping is not None:
+        rank = q_lat.shape[2]
+        c = latent[:, :rank].float()
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        kr = rotate_half_first(latent[:, rank:].float(), positions[:t], inv_freq, rot_scale)
+        row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+        bs = cache.shape[2]
+        valid = slot_mapping[:t] >= 0
+        sm = slot_mapping[:t][valid].long()
+        cache[sm // bs, 0, sm % bs, :] = row[valid]
+    return out
+
+
+def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                         token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, rank: int) -> torch.Tensor:
+    """``q[T, H, DK]`` against ``cache[blocks, 1, block, DK]``: token ``t`` reads block-table row ``token_seq[t]``
+    (``t`` itself when None) and sees keys ``0 .. seq_lens[t] - 1``; a key row's first ``rank`` values are also its
+    value.  Scores, softmax and the weighted sum in fp32; returns ``[T, H, rank]`` in ``q``'s dtype."""
+    t, hq, dk = q.shape
+    bs = cache.shape[2]
+    res = torch.zeros((t, hq, rank), dtype=torch.float32, device=q.device)
+    rows = token_seq[:t].long() if token_seq is not None else torch.arange(t, device=q.device)
+    lens = seq_lens[:t].long()
+    for b in torch.unique(rows).tolist():
+        mine = torch.nonzero(rows == b).flatten()
+        n = int(lens[mine].max())
+        if n == 0:
+            continue
+        blocks = block_table[b, :(n + bs - 1) // bs].long()
+        keys = cache[blocks, 0].reshape(-1, dk)[:n].float()
+        s = torch.einsum("thd,nd->thn", q[mine].float(), keys) * scale
+        mask = torch.arange(n, device=q.device)[None, None, :] >= lens[mine][:, None, None]
+        p = torch.softmax(s.masked_fill(mask, float("-inf")), dim=-1)
+        res[mine] = torch.einsum("thn,nd->thd", p, keys[:, :rank])
+    return res.to(q.dtype)

@@ -323,8 +323,12 @@ class ModelRunner:
 
     def get_kv_cache_spec(self) -> KVCacheSpec:
         layers = self.model.attention_layers()
-        a = layers[0]
         fp8 = self.vllm_config.cache_config.kv_fp8
+        if not layers:          # every layer recurrent: the blocks only count positions, the state is all there is
+            return KVCacheSpec(num_layers=0, num_kv_heads=0, head_dim=0, block_size=self.block_size,
+                               dtype_bytes=self.model_config.dtype_bytes, values_per_token=0,
+                               state_bytes_per_request=self._state_bytes_per_slot())
+        a = layers[0]
         windows = [int(getattr(l, "window", 0) or 0) for l in layers]
         dtype_bytes = 1 if fp8 else self.model_config.dtype_bytes
         if self.draft is not None:        # the draft reads every key it ever wrote unless it is windowed too
@@ -337,7 +341,7 @@ class ModelRunner:
         # layers of unlike shape (each with its own heads and key / value sizes): the sum over the layers is stated
         per_token = sum(l.kv_values_per_token() for l in layers)
         uniform = per_token == 2 * len(layers) * heads * width
-        state = sum(l.state_values_per_slot() for l in self._state_layers()) * self.model_config.dtype_bytes
+        state = self._state_bytes_per_slot()
         return KVCacheSpec(num_layers=len(layers), num_kv_heads=heads, head_dim=width,
                            block_size=self.block_size, dtype_bytes=dtype_bytes,
                            sliding_window=max(windows) if windows and min(windows) > 0 else None,
@@ -346,6 +350,14 @@ class ModelRunner:
                            state_bytes_per_request=state,
                            extra_bytes_per_block=(self.draft.kv_bytes_per_block(self.block_size, dtype_bytes)
                                                   if self.draft is not None else 0))
+
+    def _state_dtype(self, layer) -> torch.dtype:
+        """Convolution tails are copies of projection outputs (model dtype); a recurrence names its own (fp32)."""
+        return getattr(layer, "state_dtype", None) or self.model_config.torch_dtype
+
+    def _state_bytes_per_slot(self) -> int:
+        return sum(l.state_values_per_slot() * torch.empty((), dtype=self._state_dtype(l)).element_size()
+                   for l in self._state_layers())
 
     def _state_layers(self) -> list:
         """Layers that keep per-request state besides the KV cache (short convolutions, recurrences)."""
@@ -396,7 +408,7 @@ class ModelRunner:
         # captured decode batches
         self.state_tensors = []
         for layer in self._state_layers():
-            st = torch.zeros(layer.state_shape(self.max_num_reqs + 1), dtype=self.model_config.torch_dtype, device=self.device)
+            st = torch.zeros(layer.state_shape(self.max_num_reqs + 1), dtype=self._state_dtype(layer), device=self.device)
             layer.bind_state(st)
             self.state_tensors.append(st)
         if self.draft is not None:
@@ -1168,7 +1180,10 @@ class ModelRunner:
         if not ops.hip_available():
             return [self.max_model_len]
         from ..ops import hip
-        hkv = self.model.attention_layers()[0].num_kv_heads
+        owners = self.model.attention_layers()
+        if not owners:
+            return [self.max_model_len]
+        hkv = owners[0].num_kv_heads
         limits = [c for c in self.CONTEXT_BUCKETS if c < self.max_model_len] + [self.max_model_len]
         keep = [limits[-1]]
         for c in reversed(limits[:-1]):
@@ -1216,9 +1231,15 @@ class ModelRunner:
         if not (cc.use_hip_graph and envs.VDAMD_USE_HIP_GRAPH):
             self.graph_fallback_reason = "disabled (enforce_eager / VDAMD_USE_HIP_GRAPH=0)"
             return
-        first = self.model.attention_layers()[0]
-        kernel_head_dim = first.head_dim      # (padded to a kernel size where needed)
-        if getattr(first, "row_cache", False):        # attention over plain row caches: its kernels take any head size
+        capturable = getattr(self.model, "decode_capturable", None)
+        if capturable is not None and not capturable():
+            self.graph_fallback_reason = "a layer of the model synchronises with the host in a decode step"
+            logger.info("hipGraph decode capture: %s; running eagerly", self.graph_fallback_reason)
+            return
+        owners = self.model.attention_layers()
+        first = owners[0] if owners else None
+        kernel_head_dim = first.head_dim if owners else 0      # (padded to a kernel size where needed)
+        if first is None or getattr(first, "row_cache", False):        # attention over plain row caches: its kernels take any head size
             kernel_ok = ops.hip_available()
         elif getattr(first, "latent", False):
             kernel_ok = ops.mla_kernel_ok(first.head_dim, first.v_dim, self.model_config.torch_dtype)
@@ -1286,7 +1307,10 @@ class ModelRunner:
         if not self.is_gpu or not ops.hip_available():
             return
         from ..ops import hip
-        attn = self.model.attention_layers()[0]
+        owners = self.model.attention_layers()
+        if not owners:
+            return
+        attn = owners[0]
         n = hip.decode_workspace_floats(max(max_bs, self.max_num_reqs), attn.num_heads, attn.head_dim,
                                         attn.num_kv_heads, self.max_model_len)
         self.decode_workspace = torch.empty(n, dtype=torch.float32, device=self.device)
