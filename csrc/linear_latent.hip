@@ -1,0 +1,483 @@
+// Kernels for models that keep an fp32 residual stream between layer norms with weight and bias and mix sequences
+// with decayed linear attention and with latent attention over one row cache, gfx950.  Compiled without fast-math:
+// norms, rotations, scores, softmax weights and the recurrence are 32-bit by definition of such a model.
+//
+//   embed_scaled             token row * scale -> fp32 residual stream
+//   layer_norm_to            (x - mean) / sqrt(var + eps) * w + b of rows of any float type, result in any
+//   add_layer_norm           residual(fp32) += y ; out = layer norm of the sum                         (one launch)
+//   decay_linear_attention   S <- decay[h] S + k v^T ; o = S^T q per head, q / k / v read (through SiLU) from a fused
+//                            projection, S (dim x vdim, fp32) kept per request slot.  A workgroup owns 64 columns of
+//                            one head's S for one sequence, in registers (4 waves x dim/4 rows each), and walks the
+//                            sequence's rows in order: prompt portions and single decoded rows are the same launch
+//   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g)
+//   clamped_glu              min(g, L) sigmoid(alpha min(g, L)) (clamp(u, -L, L) + 1) over [g | u]
+//   relu_squared             max(x, 0)^2
+//   latent_prep              per token: RMS norm of the latent and rotation of the shared key part into the row cache;
+//                            the query [q_lat | rotated q_rope] assembled; angles = position * frequency in fp32
+//   latent_row_attention     causal softmax attention of every head over the shared rows (value = a row's first
+//                            `rank` values): one wave per (token, head), a lane per key for the scores, lanes over
+//                            the value's columns for the weighted sum, online softmax; any sizes, any float type
+#include "common.h"
+#include <math.h>
+#include <type_traits>
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
+
+template <typename F> int by_dtype(int dt, F&& f) {
+  switch (dt) {
+    case DT_BF16: f((bf16_t*)nullptr); return 0;
+    case DT_F16: f((f16_t*)nullptr); return 0;
+    case DT_F32: f((float*)nullptr); return 0;
+  }
+  return 1;
+}
+
+int row_threads(int h) { return h >= 2048 ? 512 : (h >= 512 ? 256 : 128); }
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+template <typename T>
+__global__ void embed_scaled_kernel(float* __restrict__ out, const int* __restrict__ ids, const T* __restrict__ embed,
+                                    float scale, int H, int vocab_rows) {
+  const long t = blockIdx.x;
+  const int id = min(max(ids[t], 0), vocab_rows - 1);
+  const T* e = embed + (long)id * H;
+  float* o = out + t * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ldf(e + i) * scale;
+}
+
+// ------------------------------------------------------------------------------------------------ layer norms
+// y == nullptr: plain norm of x (type TX, row stride x_stride).  Otherwise x is the fp32 residual stream, updated in
+// place to x + y before it is normed.
+template <typename TX, typename TY, typename TO>
+__global__ void layer_norm_kernel(TO* __restrict__ out, TX* __restrict__ x, long x_stride, const TY* __restrict__ y,
+                                  long y_stride, const float* __restrict__ w, const float* __restrict__ b, float eps,
+                                  int H) {
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  TX* xr = x + row * x_stride;
+  float sum = 0.f;
+  if (y != nullptr) {
+    if constexpr (std::is_same_v<TX, float>) {
+      const TY* yr = y + row * y_stride;
+      for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float r = xr[i] + ldf(yr + i);
+        xr[i] = r;                                         // (each thread rereads only its own stores below)
+        sum += r;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) sum += ldf(xr + i);
+  }
+  const float mean = block_sum(sum, red) / (float)H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) { const float d = ldf(xr + i) - mean; ss += d * d; }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+  TO* orow = out + row * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    stf(orow + i, (ldf(xr + i) - mean) * inv * w[i] + (b != nullptr ? b[i] : 0.f));
+}
+
+template <typename TG, typename TO>
+__global__ void gated_rms_norm_kernel(TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ w,
+                                      const TG* __restrict__ gate, long gate_stride, float eps, int N) {
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const float* orow = o + row * (long)N;
+  const TG* g = gate + row * gate_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) { const float f = orow[i]; ss += f * f; }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)N + eps);
+  TO* dst = out + row * (long)N;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)));
+}
+
+// ------------------------------------------------------------------------------------------------ activations
+template <typename T>
+__global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ h, long h_stride, int F, float limit,
+                                   float alpha) {
+  const long row = blockIdx.x;
+  const T* hr = h + row * h_stride;
+  T* o = out + row * (long)F;
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < F; i += gridDim.y * blockDim.x) {
+    const float g = fminf(ldf(hr + i), limit);
+    const float u = fminf(fmaxf(ldf(hr + F + i), -limit), limit);
+    stf(o + i, g * sigmoid_f(alpha * g) * (u + 1.0f));
+  }
+}
+
+template <typename T>
+__global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ x, long n) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const float f = fmaxf(ldf(x + i), 0.f);
+    stf(out + i, f * f);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ linear attention
+// grid (sequences, heads, column tiles of 64), 256 threads: thread (g = tid / 64, c = tid % 64) owns rows
+// g * R .. g * R + R - 1 of column c of the head's state.  x rows hold [q (H * dim) | k (H * dim) | v (H * vdim) | ..].
+// One barrier per row: q / k of the row are staged in LDS (double-buffered), the four row groups' partial outputs of
+// the previous row are summed after the next barrier.
+template <typename T, int R>
+__global__ __launch_bounds__(256) void decay_linear_attention_kernel(
+    float* __restrict__ out, const T* __restrict__ x, long x_stride, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ qsl,
+    const int* __restrict__ seq_lens, int H, int dim, int vdim, int silu) {
+  __shared__ float qs[2][4 * R], ks[2][4 * R], part[2][4][64];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, g = tid >> 6, lane = tid & 63;
+  const int c = blockIdx.z * 64 + lane;
+  const bool col = c < vdim;
+  const int s = qsl[b], e = qsl[b + 1];
+  if (e <= s) return;                                            // (uniform over the workgroup)
+  const int start = seq_lens[b] - (e - s);
+  float* st = state + ((long)slots[b] * H + h) * (long)dim * vdim;
+  const float d = decay[h];
+  float S[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int r = g * R + i;
+    S[i] = (start > 0 && col && r < dim) ? st[(long)r * vdim + c] : 0.f;
+  }
+  const long qoff = (long)h * dim, koff = (long)(H + h) * dim, voff = 2L * H * dim + (long)h * vdim + c;
+  auto act = [&](float f) { return silu ? f * sigmoid_f(f) : f; };
+  // rows beyond `dim` of the staging buffers stay zero
+  for (int i = tid; i < 4 * R; i += 256) { qs[0][i] = qs[1][i] = ks[0][i] = ks[1][i] = 0.f; }
+  float nq = 0.f, nk = 0.f, nv = 0.f;
+  {
+    const T* xr = x + (long)s * x_stride;
+    if (tid < dim) { nq = act(ldf(xr + qoff + tid)); nk = act(ldf(xr + koff + tid)); }
+    if (col) nv = act(ldf(xr + voff));
+  }
+  __syncthreads();
+  for (int r = s; r < e; ++r) {
+    const int buf = (r - s) & 1;
+    if (tid < dim) { qs[buf][tid] = nq; ks[buf][tid] = nk; }
+    const float v = nv;
+    if (r + 1 < e) {
+      const T* xr = x + (long)(r + 1) * x_stride;
+      if (tid < dim) { nq = act(ldf(xr + qoff + tid)); nk = act(ldf(xr + koff + tid)); }
+      if (col) nv = act(ldf(xr + voff));
+    }
+    __syncthreads();
+    if (r > s && g == 0 && col)
+      out[(long)(r - 1) * H * vdim + (long)h * vdim + c] =
+          (part[buf ^ 1][0][lane] + part[buf ^ 1][1][lane]) + (part[buf ^ 1][2][lane] + part[buf ^ 1][3][lane]);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      S[i] = d * S[i] + ks[buf][g * R + i] * v;
+      acc += S[i] * qs[buf][g * R + i];
+    }
+    part[buf][g][lane] = acc;
+  }
+  __syncthreads();
+  const int last = (e - 1 - s) & 1;
+  if (g == 0 && col)
+    out[(long)(e - 1) * H * vdim + (long)h * vdim + c] =
+        (part[last][0][lane] + part[last][1][lane]) + (part[last][2][lane] + part[last][3][lane]);
+  if (col) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int r = g * R + i;
+      if (r < dim) st[(long)r * vdim + c] = S[i];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent attention
+__device__ __forceinline__ void rotate_pair(float u, float v, int pos, float freq, float rs, float& ou, float& ov) {
+  const float a = (float)pos * freq;
+  const float cs = cosf(a) * rs, sn = sinf(a) * rs;
+  ou = u * cs - v * sn;
+  ov = v * cs + u * sn;
+}
+
+// one workgroup per token.  q [T, H, nope + rope] (strides q_st, q_sh), q_lat [H, T, rank] (strides l_sh, l_st),
+// latent [T, rank + rope] (stride lat_st) or nullptr, out [T, H, rank + rope] contiguous, cache rows of rank + rope.
+template <typename T>
+__global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q, long q_st, long q_sh, int nope,
+                                   const T* __restrict__ q_lat, long l_sh, long l_st, const T* __restrict__ latent,
+                                   long lat_st, const float* __restrict__ norm_w, float eps,
+                                   const float* __restrict__ inv_freq, int half, float rs,
+                                   const int* __restrict__ positions, T* __restrict__ cache,
+                                   const int* __restrict__ slot_mapping, int H, int rank, int rope) {
+  __shared__ float red[17];
+  const long t = blockIdx.x;
+  const int pos = positions[t];
+  const int dk = rank + rope;
+  T* o = out + t * (long)H * dk;
+  for (int i = threadIdx.x; i < H * rank; i += blockDim.x) {
+    const int h = i / rank, j = i - h * rank;
+    o[(long)h * dk + j] = q_lat[h * l_sh + t * l_st + j];
+  }
+  for (int i = threadIdx.x; i < H * rope; i += blockDim.x) {
+    const int h = i / rope, j = i - h * rope;
+    const T* src = q + t * q_st + h * q_sh + nope;
+    float val;
+    if (j < 2 * half) {
+      const int p = j < half ? j : j - half;
+      float a, bb;
+      rotate_pair(ldf(src + p), ldf(src + p + half), pos, inv_freq[p], rs, a, bb);
+      val = j < half ? a : bb;
+    } else {
+      val = ldf(src + j);
+    }
+    stf(o + (long)h * dk + rank + j, val);
+  }
+  if (latent == nullptr) return;                            // (uniform)
+  const T* lr = latent + t * lat_st;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float f = ldf(lr + i); ss += f * f; }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)rank + eps);
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  T* row = cache + (long)slot * dk;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) stf(row + i, ldf(lr + i) * inv * norm_w[i]);
+  for (int j = threadIdx.x; j < rope; j += blockDim.x) {
+    float val;
+    if (j < 2 * half) {
+      const int p = j < half ? j : j - half;
+      float a, bb;
+      rotate_pair(ldf(lr + rank + p), ldf(lr + rank + p + half), pos, inv_freq[p], rs, a, bb);
+      val = j < half ? a : bb;
+    } else {
+      val = ldf(lr + rank + j);
+    }
+    stf(row + rank + j, val);
+  }
+}
+
+template <typename T> __device__ __forceinline__ float dot_row(const float* __restrict__ qs, const T* __restrict__ k, int dk) {
+  float acc = 0.f;
+  if constexpr (std::is_same_v<T, float>) {
+    if ((dk & 3) == 0) {
+      for (int d = 0; d < dk; d += 4) {
+        const float4 kv = *reinterpret_cast<const float4*>(k + d);
+        acc += qs[d] * kv.x; acc += qs[d + 1] * kv.y; acc += qs[d + 2] * kv.z; acc += qs[d + 3] * kv.w;
+      }
+      return acc;
+    }
+  } else {
+    if ((dk & 7) == 0) {
+      for (int d = 0; d < dk; d += 8) {
+        const typename Vec8<T>::type kv = ld8<T>(k + d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += qs[d + e] * (float)kv[e];
+      }
+      return acc;
+    }
+  }
+  for (int d = 0; d < dk; ++d) acc += qs[d] * ldf(k + d);
+  return acc;
+}
+
+// grid (tokens, ceil(H / 4)), 256 threads: wave w serves head blockIdx.y * 4 + w.  Waves share nothing but the
+// workgroup's LDS allocation (each its own query copy): no workgroup barrier.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void latent_row_attention_kernel(
+    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
+    long bt_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_lens, float scale, int H, int dk,
+    int rank, int bs) {
+  extern __shared__ float q_lds[];
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long t = blockIdx.x;
+  const int h = blockIdx.y * 4 + w;
+  if (h >= H) return;
+  float* qs = q_lds + (long)w * dk;
+  const T* qr = q + (t * H + h) * (long)dk;
+  for (int d = lane; d < dk; d += 64) qs[d] = ldf(qr + d);
+  __builtin_amdgcn_wave_barrier();
+  const int n = seq_lens[t];
+  const int* bt = block_table + (token_seq != nullptr ? (long)token_seq[t] : t) * bt_stride;
+  float m = -1.0e30f, l = 0.f;
+  float o[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) o[i] = 0.f;
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    const bool valid = j < n;
+    long row = 0;
+    float sc = -1.0e30f;
+    if (valid) {
+      row = ((long)bt[j / bs] * bs + (j % bs)) * dk;
+      sc = dot_row<T>(qs, cache + row, dk) * scale;
+    }
+    const float m_new = fmaxf(m, wave_max(sc));
+    const float p = valid ? expf(sc - m_new) : 0.f;
+    const float alpha = expf(m - m_new);
+    l = l * alpha + wave_sum(p);
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) o[i] *= alpha;
+    const int cnt = min(64, n - j0);
+    const int row_lo = (int)(row & 0xffffffffL), row_hi = (int)(row >> 32);
+    for (int jj = 0; jj < cnt; ++jj) {
+      const float pj = __shfl(p, jj, 64);
+      const long ro = ((long)__shfl(row_hi, jj, 64) << 32) | (unsigned int)__shfl(row_lo, jj, 64);
+      const T* vr = cache + ro;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int dcol = lane + 64 * i;
+        if (dcol < rank) o[i] += pj * ldf(vr + dcol);
+      }
+    }
+  }
+  T* orow = out + (t * H + h) * (long)rank;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int dcol = lane + 64 * i;
+    if (dcol < rank) stf(orow + dcol, o[i] * inv);
+  }
+}
+
+}  // namespace
+
+VDAMD_API int vdamd_embed_scaled(float* out, const int* ids, const void* embed, float scale, int T, int H,
+                                 int vocab_rows, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || vocab_rows <= 0) return 1;
+  return by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((embed_scaled_kernel<TT>), dim3(T), dim3(row_threads(H)), 0, stream, out, ids, (const TT*)embed,
+                       scale, H, vocab_rows);
+  });
+}
+
+// y == nullptr: out = LN(x) with x of type x_dt.  Otherwise x is the fp32 residual (x_dt must be DT_F32, x_stride H).
+VDAMD_API int vdamd_layer_norm_to(void* out, void* x, long x_stride, const void* y, long y_stride, const float* w,
+                                  const float* b, float eps, int rows, int H, int x_dt, int y_dt, int out_dt,
+                                  hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || w == nullptr || (y != nullptr && x_dt != DT_F32)) return 1;
+  const int th = row_threads(H);
+  int i1 = 0, i2 = 0;
+  const int rc = by_dtype(x_dt, [&](auto* tx) {
+    using TX = std::remove_pointer_t<decltype(tx)>;
+    i1 = by_dtype(y_dt, [&](auto* ty) {
+      using TY = std::remove_pointer_t<decltype(ty)>;
+      i2 = by_dtype(out_dt, [&](auto* to) {
+        using TO = std::remove_pointer_t<decltype(to)>;
+        hipLaunchKernelGGL((layer_norm_kernel<TX, TY, TO>), dim3(rows), dim3(th), 0, stream, (TO*)out, (TX*)x, x_stride,
+                           (const TY*)y, y_stride, w, b, eps, H);
+      });
+    });
+  });
+  if (rc | i1 | i2) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+VDAMD_API int vdamd_gated_rms_norm(void* out, const float* o, const float* w, const void* gate, long gate_stride,
+                                   float eps, int rows, int N, int gate_dt, int out_dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (N <= 0) return 1;
+  int inner = 0;
+  const int rc = by_dtype(gate_dt, [&](auto* tg) {
+    using TG = std::remove_pointer_t<decltype(tg)>;
+    inner = by_dtype(out_dt, [&](auto* to) {
+      using TO = std::remove_pointer_t<decltype(to)>;
+      hipLaunchKernelGGL((gated_rms_norm_kernel<TG, TO>), dim3(rows), dim3(row_threads(N)), 0, stream, (TO*)out, o, w,
+                         (const TG*)gate, gate_stride, eps, N);
+    });
+  });
+  if (rc | inner) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+VDAMD_API int vdamd_clamped_glu(void* out, const void* h, long h_stride, int rows, int F, float limit, float alpha,
+                                int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (F <= 0) return 1;
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((clamped_glu_kernel<TT>), dim3(rows, (F + 1023) / 1024), dim3(256), 0, stream, (TT*)out,
+                       (const TT*)h, h_stride, F, limit, alpha);
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+VDAMD_API int vdamd_relu_squared(void* out, const void* x, long n, int dt, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const unsigned blocks = (unsigned)((n + 1023) / 1024 > 65535 ? 65535 : (n + 1023) / 1024);
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((relu_squared_kernel<TT>), dim3(blocks), dim3(256), 0, stream, (TT*)out, (const TT*)x, n);
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+// x [T, x_stride] of type dt, out fp32 [T, H * vdim], state fp32 [slots, H, dim, vdim]; dim <= 256
+VDAMD_API int vdamd_decay_linear_attention(float* out, const void* x, long x_stride, const float* decay, float* state,
+                                           const int* slots, const int* qsl, const int* seq_lens, int num_seqs, int H,
+                                           int dim, int vdim, int silu, int dt, hipStream_t stream) {
+  if (num_seqs <= 0) return 0;
+  if (H <= 0 || dim <= 0 || vdim <= 0 || dim > 256) return 1;
+  const dim3 grid(num_seqs, H, (vdim + 63) / 64);
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+#define DLA(R_)                                                                                                      \
+  hipLaunchKernelGGL((decay_linear_attention_kernel<TT, R_>), grid, dim3(256), 0, stream, out, (const TT*)x, x_stride, \
+                     decay, state, slots, qsl, seq_lens, H, dim, vdim, silu)
+    if (dim <= 32) DLA(8);
+    else if (dim <= 64) DLA(16);
+    else if (dim <= 128) DLA(32);
+    else DLA(64);
+#undef DLA
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+VDAMD_API int vdamd_latent_prep(void* out, const void* q, long q_st, long q_sh, int nope, const void* q_lat, long l_sh,
+                                long l_st, const void* latent, long lat_st, const float* norm_w, float eps,
+                                const float* inv_freq, int half, float rs, const int* positions, void* cache,
+                                const int* slot_mapping, int T, int H, int rank, int rope, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || rank <= 0 || rope < 0 || 2 * half > rope) return 1;
+  if (latent != nullptr && (cache == nullptr || slot_mapping == nullptr || norm_w == nullptr)) return 1;
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((latent_prep_kernel<TT>), dim3(T), dim3(256), 0, stream, (TT*)out, (const TT*)q, q_st, q_sh, nope,
+                       (const TT*)q_lat, l_sh, l_st, (const TT*)latent, lat_st, norm_w, eps, inv_freq, half, rs,
+                       positions, (TT*)cache, slot_mapping, H, rank, rope);
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+VDAMD_API int vdamd_latent_row_attention(void* out, const void* q, const void* cache, const int* block_table,
+                                         long bt_stride, const int* token_seq, const int* seq_lens, float scale, int T,
+                                         int H, int dk, int rank, int bs, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || rank <= 0 || rank > dk || dk > 4096 || rank > 1024 || bs <= 0) return 1;
+  const dim3 grid(T, (H + 3) / 4);
+  const size_t lds = (size_t)4 * dk * sizeof(float);
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+#define LRA(NV_)                                                                                                      \
+  hipLaunchKernelGGL((latent_row_attention_kernel<TT, NV_>), grid, dim3(256), lds, stream, (TT*)out, (const TT*)q,     \
+                     (const TT*)cache, block_table, bt_stride, token_seq, seq_lens, scale, H, dk, rank, bs)
+    if (rank <= 64) LRA(1);
+    else if (rank <= 128) LRA(2);
+    else if (rank <= 256) LRA(4);
+    else if (rank <= 512) LRA(8);
+    else LRA(16);
+#undef LRA
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}

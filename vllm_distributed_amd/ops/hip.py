@@ -70,6 +70,14 @@ def load() -> ctypes.CDLL:
         "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
         "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, I, P],
         "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, P],
+        "vdamd_embed_scaled": [P, P, P, F, I, I, I, I, P],
+        "vdamd_layer_norm_to": [P, P, L, P, L, P, P, F, I, I, I, I, I, P],
+        "vdamd_gated_rms_norm": [P, P, P, P, L, F, I, I, I, I, P],
+        "vdamd_clamped_glu": [P, P, L, I, I, F, F, I, P],
+        "vdamd_relu_squared": [P, P, L, I, P],
+        "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, P],
+        "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, I, I, I, I, I, P],
+        "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -1351,4 +1359,131 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, b, h, g, d, dv, bs,
         int(window), int(keep_first), int(max_query_len) if max_query_len else t, float(scale), float(softcap),
         1 if WINDOW_ATTENTION_MFMA else 0, _dt(q), _stream()), "window_bias_attention")
+    return out
+
+
+# ------------------------------------------------ fp32 residual stream with layer norms, decayed linear attention,
+# ------------------------------------------------ gated norm, clamped GLU, latent attention over one row cache
+def embed_scaled(ids: torch.Tensor, weight: torch.Tensor, scale: float) -> torch.Tensor:
+    t, h = ids.numel(), weight.shape[1]
+    assert ids.dtype == torch.int32 and weight.is_contiguous()
+    out = torch.empty((t, h), dtype=torch.float32, device=weight.device)
+    _check(_LIB.vdamd_embed_scaled(out.data_ptr(), ids.data_ptr(), weight.data_ptr(), float(scale), t, h,
+                                   weight.shape[0], _dt(weight), _stream()), "embed_scaled")
+    return out
+
+
+def layer_norm_to(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    t, h = x.shape
+    assert x.stride(1) == 1
+    out = torch.empty((t, h), dtype=out_dtype, device=x.device)
+    _check(_LIB.vdamd_layer_norm_to(out.data_ptr(), x.data_ptr(), x.stride(0), None, 0,
+                                    _f32_vec(weight, h, "weight").data_ptr(), _ptr(_f32_vec(bias, h, "bias")),
+                                    float(eps), t, h, _dt(x), _dt(x), _DT[out_dtype], _stream()), "layer_norm_to")
+    return out
+
+
+def add_layer_norm(y: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                   eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    t, h = y.shape
+    assert residual.shape == (t, h) and residual.dtype == torch.float32 and residual.is_contiguous() and y.stride(1) == 1
+    out = torch.empty((t, h), dtype=out_dtype, device=y.device)
+    _check(_LIB.vdamd_layer_norm_to(out.data_ptr(), residual.data_ptr(), h, y.data_ptr(), y.stride(0),
+                                    _f32_vec(weight, h, "weight").data_ptr(), _ptr(_f32_vec(bias, h, "bias")),
+                                    float(eps), t, h, _DT[torch.float32], _dt(y), _DT[out_dtype], _stream()),
+           "add_layer_norm")
+    return out
+
+
+DECAY_ATTENTION_MAX_DIM = 256
+
+
+def decay_linear_attention(x: torch.Tensor, num_heads: int, dim: int, vdim: int, decay: torch.Tensor,
+                           state: torch.Tensor, slots: torch.Tensor, query_start_loc: torch.Tensor,
+                           seq_lens: torch.Tensor, silu: bool = True, max_query_len: int = 0) -> torch.Tensor:
+    t = x.shape[0]
+    n = seq_lens.numel()
+    if dim > DECAY_ATTENTION_MAX_DIM:
+        raise NotImplementedError(f"decayed linear attention with key size {dim} > {DECAY_ATTENTION_MAX_DIM}")
+    assert x.stride(1) == 1 and x.shape[1] >= num_heads * (2 * dim + vdim)
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (num_heads, dim, vdim)
+    assert slots.dtype == seq_lens.dtype == query_start_loc.dtype == torch.int32
+    assert slots.numel() >= n and query_start_loc.numel() >= n + 1
+    out = torch.empty((t, num_heads * vdim), dtype=torch.float32, device=x.device)
+    _check(_LIB.vdamd_decay_linear_attention(out.data_ptr(), x.data_ptr(), x.stride(0),
+                                             _f32_vec(decay, num_heads, "decay").data_ptr(), state.data_ptr(),
+                                             slots.data_ptr(), query_start_loc.data_ptr(), seq_lens.data_ptr(), n,
+                                             num_heads, dim, vdim, int(bool(silu)), _dt(x), _stream()),
+           "decay_linear_attention")
+    return out
+
+
+def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    t, n = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and gate.shape == (t, n) and gate.stride(1) == 1
+    out = torch.empty((t, n), dtype=out_dtype, device=o.device)
+    _check(_LIB.vdamd_gated_rms_norm(out.data_ptr(), o.data_ptr(), _f32_vec(weight, n, "weight").data_ptr(),
+                                     gate.data_ptr(), gate.stride(0), float(eps), t, n, _dt(gate), _DT[out_dtype],
+                                     _stream()), "gated_rms_norm")
+    return out
+
+
+def clamped_glu(h: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    f = h.shape[-1] // 2
+    h2 = h.reshape(-1, 2 * f)
+    if h2.stride(1) != 1:
+        h2 = h2.contiguous()
+    out = torch.empty((h2.shape[0], f), dtype=h.dtype, device=h.device)
+    _check(_LIB.vdamd_clamped_glu(out.data_ptr(), h2.data_ptr(), h2.stride(0), h2.shape[0], f, float(limit),
+                                  float(alpha), _dt(h2), _stream()), "clamped_glu")
+    return out.view(h.shape[:-1] + (f,))
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    xc = x if x.is_contiguous() else x.contiguous()
+    out = torch.empty_like(xc)
+    _check(_LIB.vdamd_relu_squared(out.data_ptr(), xc.data_ptr(), xc.numel(), _dt(xc), _stream()), "relu_squared")
+    return out
+
+
+def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
+                norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
+                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> torch.Tensor:
+    t, h, qd = q.shape
+    rank, rope = q_lat.shape[2], qd - nope
+    half = inv_freq.numel()
+    assert q.stride(2) == 1 and q_lat.stride(2) == 1 and q_lat.shape == (h, t, rank) and q_lat.dtype == q.dtype
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and 2 * half <= rope
+    assert positions.dtype == torch.int32 and positions.numel() >= t
+    out = torch.empty((t, h, rank + rope), dtype=q.dtype, device=q.device)
+    write = latent is not None and cache is not None and slot_mapping is not None
+    if write:
+        assert latent.shape == (t, rank + rope) and latent.stride(1) == 1 and latent.dtype == q.dtype
+        assert cache.is_contiguous() and cache.dtype == q.dtype and cache.shape[1] == 1 and cache.shape[3] == rank + rope
+        assert slot_mapping.dtype == torch.int32 and slot_mapping.numel() >= t
+    _check(_LIB.vdamd_latent_prep(
+        out.data_ptr(), q.data_ptr(), q.stride(0), q.stride(1), nope, q_lat.data_ptr(), q_lat.stride(0),
+        q_lat.stride(1), latent.data_ptr() if write else None, latent.stride(0) if write else 0,
+        _f32_vec(norm_weight, rank, "norm_weight").data_ptr() if write else None, float(eps), inv_freq.data_ptr(),
+        half, float(rot_scale), positions.data_ptr(), cache.data_ptr() if write else None,
+        slot_mapping.data_ptr() if write else None, t, h, rank, rope, _dt(q), _stream()), "latent_prep")
+    return out
+
+
+def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                         token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, rank: int,
+                         max_seq_len: int = 0) -> torch.Tensor:
+    t, h, dk = q.shape
+    assert q.is_contiguous() and cache.is_contiguous() and cache.dtype == q.dtype
+    assert cache.shape[1] == 1 and cache.shape[3] == dk and 0 < rank <= dk
+    assert block_table.dtype == torch.int32 and block_table.stride(1) == 1 and seq_lens.dtype == torch.int32
+    assert seq_lens.numel() >= t and (token_seq is None or (token_seq.dtype == torch.int32 and token_seq.numel() >= t))
+    assert token_seq is not None or block_table.shape[0] >= t
+    out = torch.empty((t, h, rank), dtype=q.dtype, device=q.device)
+    _check(_LIB.vdamd_latent_row_attention(out.data_ptr(), q.data_ptr(), cache.data_ptr(), block_table.data_ptr(),
+                                           block_table.stride(0), None if token_seq is None else token_seq.data_ptr(),
+                                           seq_lens.data_ptr(), float(scale), t, h, dk, rank, cache.shape[2], _dt(q),
+                                           _stream()), "latent_row_attention")
     return out
