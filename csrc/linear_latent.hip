@@ -204,8 +204,8 @@ __global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q,
                                    const T* __restrict__ q_lat, long l_sh, long l_st, const T* __restrict__ latent,
                                    long lat_st, const float* __restrict__ norm_w, float eps,
                                    const float* __restrict__ inv_freq, int half, float rs,
-                                   const int* __restrict__ positions, T* __restrict__ cache,
-                                   const int* __restrict__ slot_mapping, int H, int rank, int rope) {
+                                   const int* __restrict__ positions, T* __restrict__ cache, T* __restrict__ vfrag,
+                                   const int* __restrict__ slot_mapping, int H, int rank, int rope, int bs) {
   __shared__ float red[17];
   const long t = blockIdx.x;
   const int pos = positions[t];
@@ -238,6 +238,15 @@ __global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q,
   if (slot < 0) return;
   T* row = cache + (long)slot * dk;
   for (int i = threadIdx.x; i < rank; i += blockDim.x) stf(row + i, ldf(lr + i) * inv * norm_w[i]);
+  if (vfrag != nullptr) {
+    // the same values as V^T fragments [blocks][rank / 16][bs / 8][16][8] (what the matrix-core kernel reads)
+    const long blk = slot / bs;
+    const int off = slot % bs;
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+      const long at = (((blk * (rank >> 4) + (i >> 4)) * (bs >> 3) + (off >> 3)) * 16 + (i & 15)) * 8 + (off & 7);
+      stf(vfrag + at, ldf(lr + i) * inv * norm_w[i]);
+    }
+  }
   for (int j = threadIdx.x; j < rope; j += blockDim.x) {
     float val;
     if (j < 2 * half) {
@@ -443,15 +452,17 @@ VDAMD_API int vdamd_decay_linear_attention(float* out, const void* x, long x_str
 VDAMD_API int vdamd_latent_prep(void* out, const void* q, long q_st, long q_sh, int nope, const void* q_lat, long l_sh,
                                 long l_st, const void* latent, long lat_st, const float* norm_w, float eps,
                                 const float* inv_freq, int half, float rs, const int* positions, void* cache,
-                                const int* slot_mapping, int T, int H, int rank, int rope, int dt, hipStream_t stream) {
+                                void* vfrag, const int* slot_mapping, int T, int H, int rank, int rope, int bs, int dt,
+                                hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || rank <= 0 || rope < 0 || 2 * half > rope) return 1;
+  if (vfrag != nullptr && (latent == nullptr || rank % 16 || bs <= 0 || bs % 8)) return 1;
   if (latent != nullptr && (cache == nullptr || slot_mapping == nullptr || norm_w == nullptr)) return 1;
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
     hipLaunchKernelGGL((latent_prep_kernel<TT>), dim3(T), dim3(256), 0, stream, (TT*)out, (const TT*)q, q_st, q_sh, nope,
                        (const TT*)q_lat, l_sh, l_st, (const TT*)latent, lat_st, norm_w, eps, inv_freq, half, rs,
-                       positions, (TT*)cache, slot_mapping, H, rank, rope);
+                       positions, (TT*)cache, (TT*)vfrag, slot_mapping, H, rank, rope, bs);
   });
   if (rc) return 1;
   HIP_LAUNCH_CHECK();

@@ -92,7 +92,9 @@ __device__ __forceinline__ void mla_st(void* cache, long off, float v) {
   }
 }
 
-template <typename T, int DK, int DV, bool KV8>
+// P2: the fp32 softmax weights enter the PV product as a high and a low 16-bit part (two MFMAs per tile, ~16
+// mantissa bits) instead of being rounded to 8 bits: for models that define their attention weights in 32-bit.
+template <typename T, int DK, int DV, bool KV8, bool P2>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void mla_attention_kernel(
     T* __restrict__ out, long out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const T* __restrict__ q, long q_stride, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
@@ -196,18 +198,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float alpha = fast_exp2(m - m_new);
     float psum = 0.f;
     V pf;
+    [[maybe_unused]] V pl;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float e = p[j] <= 0.5f * MLA_NEG_BIG ? 0.f : fast_exp2(p[j] - m_new);
       psum += e;
       pf[j] = (T)e;
+      if constexpr (P2) pl[j] = (T)(e - (float)pf[j]);
     }
     l = l * alpha + psum;
     m = m_new;
 #pragma unroll
     for (int i = 0; i < VT; ++i) {
       acc[i] *= alpha;
-      acc[i] = mfma16(mla_widen<T, KV8>(cur.vf[i]), pf, acc[i]);
+      const V vfrag = mla_widen<T, KV8>(cur.vf[i]);
+      acc[i] = mfma16(vfrag, pf, acc[i]);
+      if constexpr (P2) acc[i] = mfma16(vfrag, pl, acc[i]);
     }
     cur = nxt;
   }
@@ -246,7 +252,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // Same split of the two reductions over the four waves; one wave per SIMD (the NQ accumulator sets and query
 // fragments take the registers the second wave had), all NQ partial score tiles exchanged behind one barrier.
 // ---------------------------------------------------------------------------------------------------------------
-template <typename T, int DK, int DV, int NQ, bool BY_TOKEN, bool KV8>
+template <typename T, int DK, int DV, int NQ, bool BY_TOKEN, bool KV8, bool P2>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mla_attention_multi_kernel(
     T* __restrict__ out, long out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const T* __restrict__ q, long q_stride, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
@@ -396,11 +402,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       const float alpha = fast_exp2(m[n] - m_new);
       float psum = 0.f;
       V pf;
+      [[maybe_unused]] V pl;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float e = p[j] <= 0.5f * MLA_NEG_BIG ? 0.f : fast_exp2(p[j] - m_new);
         psum += e;
         pf[j] = (T)e;
+        if constexpr (P2) pl[j] = (T)(e - (float)pf[j]);
       }
       l[n] = l[n] * alpha + psum;
       m[n] = m_new;
@@ -408,6 +416,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int i = 0; i < VT; ++i) {
         acc[n][i] *= alpha;
         acc[n][i] = mfma16(vf[i], pf, acc[n][i]);
+        if constexpr (P2) acc[n][i] = mfma16(vf[i], pl, acc[n][i]);
       }
     }
     cur = nxt;
@@ -531,7 +540,7 @@ __global__ __launch_bounds__(256) void mla_prep_kernel(
   }
 }
 
-template <typename T, int DK, int DV, bool KV8>
+template <typename T, int DK, int DV, bool KV8, bool P2>
 int launch_mla(void* out, long out_stride, void* part_o, void* part_ml, const void* q, long q_stride,
                const void* k_cache, const void* v_cache, const int* block_table, int bt_stride, const int* token_seq,
                const int* seq_lens, float scale, int T_, int Hq, int block_size, int num_splits, int mode,
@@ -541,15 +550,15 @@ int launch_mla(void* out, long out_stride, void* part_o, void* part_ml, const vo
   constexpr int NQ = 4;
   if (mode == 1 && token_seq != nullptr) {          // NQ consecutive tokens of a sequence share the cache stream
     // (ids walk the tokens residue class by residue class: (T_ + NQ - 1) / NQ ids per class)
-    mla_attention_multi_kernel<T, DK, DV, NQ, true, KV8><<<dim3(num_splits, q_tiles, (T_ + NQ - 1) / NQ * NQ), 256, 0, st>>>(
+    mla_attention_multi_kernel<T, DK, DV, NQ, true, KV8, P2><<<dim3(num_splits, q_tiles, (T_ + NQ - 1) / NQ * NQ), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
         bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits);
   } else if (mode == 2) {                           // NQ head tiles of a token share it
-    mla_attention_multi_kernel<T, DK, DV, NQ, false, KV8><<<dim3(num_splits, (q_tiles + NQ - 1) / NQ, T_), 256, 0, st>>>(
+    mla_attention_multi_kernel<T, DK, DV, NQ, false, KV8, P2><<<dim3(num_splits, (q_tiles + NQ - 1) / NQ, T_), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
         bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits);
   } else {
-    mla_attention_kernel<T, DK, DV, KV8><<<dim3(num_splits, q_tiles, T_), 256, 0, st>>>(
+    mla_attention_kernel<T, DK, DV, KV8, P2><<<dim3(num_splits, q_tiles, T_), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
         bt_stride, token_seq, seq_lens, sl2, Hq, block_size, num_splits);
   }
@@ -566,16 +575,21 @@ template <typename T>
 int dispatch_mla(int DK, int DV, int kv_fp8, void* out, long out_stride, void* part_o, void* part_ml, const void* q,
                  long q_stride, const void* k_cache, const void* v_cache, const int* block_table, int bt_stride,
                  const int* token_seq, const int* seq_lens, float scale, int T_, int Hq, int block_size,
-                 int num_splits, int mode, hipStream_t st) {
+                 int num_splits, int mode, int precise, hipStream_t st) {
+  if (precise && kv_fp8) return -6;       // (split weights over an 8-bit cache: not built)
 #define MLA_CASE(DK_, DV_)                                                                                        \
   if (DK == DK_ && DV == DV_) {                                                                                   \
     if (kv_fp8)                                                                                                   \
-      return launch_mla<T, DK_, DV_, true>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,       \
-                                           block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, \
-                                           num_splits, mode, st);                                                 \
-    return launch_mla<T, DK_, DV_, false>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,        \
-                                          block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, \
-                                          num_splits, mode, st);                                                  \
+      return launch_mla<T, DK_, DV_, true, false>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
+                                                  block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,     \
+                                                  block_size, num_splits, mode, st);                              \
+    if (precise)                                                                                                  \
+      return launch_mla<T, DK_, DV_, false, true>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
+                                                  block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,     \
+                                                  block_size, num_splits, mode, st);                              \
+    return launch_mla<T, DK_, DV_, false, false>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
+                                                 block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,      \
+                                                 block_size, num_splits, mode, st);                               \
   }
   MLA_CASE(576, 512) MLA_CASE(96, 64) MLA_CASE(320, 256)
 #undef MLA_CASE
@@ -594,7 +608,7 @@ VDAMD_API int vdamd_mla_attention(void* out, long out_stride, void* part_o, void
                                   long q_stride, const void* k_cache, const void* v_cache, const int* block_table,
                                   int bt_stride, const int* token_seq, const int* seq_lens, float scale, int T_,
                                   int Hq, int DK, int DV, int block_size, int num_splits, int mode, int dtype,
-                                  int kv_fp8, void* stream) {
+                                  int kv_fp8, int precise, void* stream) {
   if (T_ <= 0) return 0;
   if (block_size % 8 || num_splits < 1 || num_splits > MLA_MAX_SPLITS) return -1;
   if (num_splits > 1 && (part_o == nullptr || part_ml == nullptr)) return -2;
@@ -603,11 +617,11 @@ VDAMD_API int vdamd_mla_attention(void* out, long out_stride, void* part_o, void
   if (dtype == DT_BF16)
     return dispatch_mla<bf16_t>(DK, DV, kv_fp8, out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,
                                 block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, num_splits,
-                                mode, st);
+                                mode, precise, st);
   if (dtype == DT_F16)
     return dispatch_mla<f16_t>(DK, DV, kv_fp8, out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,
                                block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, num_splits,
-                               mode, st);
+                               mode, precise, st);
   return -3;
 }
 

@@ -121,28 +121,38 @@ def glu_expert(h, w, p, limit, alpha=1.702):
     return (g * sigmoid(alpha * g) * (u + 1)) @ f64(w[p + "down"]).T
 
 
-def route(z, correction, top, groups, keep):
-    """Router logits ``z [T, n]`` -> (chosen outputs ``[T, top]``, their weights)."""
+def route(z, correction, top, groups, keep, margins=None):
+    """Router logits ``z [T, n]`` -> (chosen outputs ``[T, top]``, their weights).  ``margins`` (a list) receives, per
+    token, by how much the choice was made: the gap between the last chosen and the first rejected choice score, and
+    between the last kept and the first dropped group."""
     n = z.shape[1]
     s = torch.softmax(z, -1)
     choice = s + f64(correction)
+    margin = torch.full((z.shape[0],), math.inf, dtype=F64)
     if groups > 1 and keep < groups:
         size = n // groups
         for t in range(z.shape[0]):
-            best = sorted(range(groups), key=lambda g: -float(choice[t, g * size:(g + 1) * size].max()))[:keep]
-            for g in range(groups):
-                if g not in best:
-                    choice[t, g * size:(g + 1) * size] = -math.inf
+            score = [float(choice[t, g * size:(g + 1) * size].max()) for g in range(groups)]
+            best = sorted(range(groups), key=lambda g: -score[g])
+            margin[t] = score[best[keep - 1]] - score[best[keep]]
+            for g in best[keep:]:
+                choice[t, g * size:(g + 1) * size] = -math.inf
+    ranked = torch.sort(choice, -1, descending=True).values
+    if top < n:
+        margin = torch.minimum(margin, ranked[:, top - 1] - ranked[:, top])
+    if margins is not None:
+        margins.append(margin)
     idx = torch.topk(choice, top, -1).indices
     wts = s.gather(1, idx)
     return idx, wts / (wts.sum(-1, keepdim=True) + 1e-20)
 
 
-def moe(h, w, p, mlp):
+def moe(h, w, p, mlp, margins=None):
     r = mlp["router"]
     experts, top = r["experts"], r["top"]
     g = r.get("groups") or {}
-    idx, wts = route(h @ f64(w[p + "router"]).T, w[p + "correction"], top, g.get("count", 1), g.get("keep", g.get("count", 1)))
+    idx, wts = route(h @ f64(w[p + "router"]).T, w[p + "correction"], top, g.get("count", 1),
+                     g.get("keep", g.get("count", 1)), margins)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(top):
@@ -159,9 +169,9 @@ def dense(h, w, p):
 
 
 # ------------------------------------------------------------------------------------------------ the model
-def forward(cfg, w, tokens, residuals=None):
+def forward(cfg, w, tokens, residuals=None, margins=None):
     """Logits ``[T, vocab]`` of one sequence from position 0; ``residuals`` (a list) collects the stream after every
-    layer."""
+    layer, ``margins`` (a list) one tensor per routed layer: see ``route``."""
     eps = cfg["norm"]["eps"]
     positions = torch.arange(len(tokens))
     x = f64(w["embed"])[torch.tensor(tokens)] * cfg["embedding"]["scale"]
@@ -177,7 +187,7 @@ def forward(cfg, w, tokens, residuals=None):
             x = x + latent_mixer(h, w, p + "mix.", m, rows[i if m.get("kv_from") is None else m["kv_from"]], positions)
         if spec.get("mlp"):
             h = layer_norm(x, w[p + "norm2"], w[p + "norm2.b"], eps)
-            x = x + (dense(h, w, p + "mlp.") if spec["mlp"].get("kind", "dense") == "dense" else moe(h, w, p + "mlp.", spec["mlp"]))
+            x = x + (dense(h, w, p + "mlp.") if spec["mlp"].get("kind", "dense") == "dense" else moe(h, w, p + "mlp.", spec["mlp"], margins))
         if residuals is not None:
             residuals.append(x.clone())
     return layer_norm(x, w["final.norm"], w["final.norm.b"], eps) @ f64(w["head"]).T

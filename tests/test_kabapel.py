@@ -4,8 +4,7 @@ GPU / reference ops on the CPU) against the plain float64 model of ``tests/kabap
 Every test builds its own small configuration and random weights (stored as bfloat16, so the oracle and the framework
 read the same numbers).  The schedules go through ``EngineCore.step_forced`` and generation goes through
 ``LLM.generate``.  The CPU tests run in float32; the GPU tests run the HIP kernels in float32 (tight tolerance: an index
-that is one off shows) and in bfloat16.  In bfloat16 the router sees a rounded input, so a near-tie between two
-experts may fall the other way than in the oracle: there a few rows (3 %) may miss the tolerance; in float32 none may.
+that is one off shows) and in bfloat16 (with routers made decisive, see ``model_dir``).
 """
 import json
 import os
@@ -78,6 +77,9 @@ CONFIGS = {
     "recurrent_only": config([lightning(2, 16, 24, [0.9, 0.95], dense(48)), lightning(4, 8, 8, [0.6, 0.7, 0.8, 0.9])], width=32),
     "attention_only": config([latent(2, 16, 8, 16, 32, 0.2, rot(8), dense(48)),
                               latent(3, 8, 8, 8, 32, 0.3, rot(8), moe(4, 2, 2, 16, 1.0, groups=(2, 1)), kv_from=0)], width=32),
+    # a latent width the matrix-core kernel is built for (64 + 32): rows and V^T fragments, shared with a reader
+    "fragments": config([latent(4, 16, 32, 16, 64, 0.2, rot(32), dense(64)), lightning(2, 32, 32, [0.9, 0.99], dense(48)),
+                         latent(3, 8, 32, 24, 64, 0.2, rot(32), moe(4, 1, 2, 32, 1.0), kv_from=0)], width=64),
     # wider, for pages of 16 tokens
     "paged": config([lightning(4, 16, 16, [0.8, 0.95, 0.99, 0.999], dense(96)),
                      latent(4, 16, 8, 16, 32, 0.2, rot(8), moe(6, 2, 2, 32, 1.0, groups=(4, 3), shared=(32, 1.0))),
@@ -137,38 +139,47 @@ def random_weights(cfg, seed):
 _MODELS = {}
 
 
-def model_dir(name, tmp_path_factory):
-    if name not in _MODELS:
+def model_dir(name, tmp_path_factory, dtype="float32"):
+    """The model's folder, configuration and weights.  For bfloat16 runs the routers are made decisive: their
+    corrections are set two apart in a random order, so that every token chooses the same outputs (identity ones
+    among them or not) whatever rounding does to the scores - the weights of the chosen still differ from token to
+    token.  In bfloat16 the router's input carries the rounding of every layer before it, and a close call that falls
+    the other way swaps a whole expert; the float32 runs keep the free-running routers."""
+    decisive = dtype != "float32"
+    if (name, decisive) not in _MODELS:
         from safetensors.torch import save_file
         cfg = CONFIGS[name]
         w = random_weights(cfg, seed=sum(map(ord, name)))
+        if decisive:
+            g = torch.Generator().manual_seed(11)
+            for k in [k for k in w if k.endswith(".correction")]:
+                w[k] = (torch.randperm(w[k].numel(), generator=g) * 2.0 - w[k].numel()).to(torch.bfloat16)
         d = tmp_path_factory.mktemp("kabapel_" + name)
         save_file({k: v.contiguous() for k, v in w.items()}, str(d / "model.safetensors"))
         (d / "config.json").write_text(json.dumps(cfg))
-        _MODELS[name] = (str(d), cfg, w)
-    return _MODELS[name]
+        _MODELS[(name, decisive)] = (str(d), cfg, w)
+    return _MODELS[(name, decisive)]
 
 
 _ORACLE = {}
 
 
 def oracle_logits(name, cfg, w, tokens):
-    key = (name, tuple(tokens))
+    key = (name, id(w), tuple(tokens))
     if key not in _ORACLE:
         _ORACLE[key] = oracle.forward(cfg, w, list(tokens)).numpy()
     return _ORACLE[key]
 
 
-def check(got, name, cfg, w, reqs, tol, dtype):
+def check(got, name, cfg, w, reqs, tol, dtype=None):
+    """Every row the run produced against the oracle."""
     assert got
-    bad = []
     for (rid, p), row in got.items():
         err = np.abs(row - oracle_logits(name, cfg, w, reqs[rid])[p]).max()
-        assert np.isfinite(err)
-        if err > tol:
-            bad.append((rid, p, float(err)))
-    allowed = 0 if dtype == "float32" else max(1, int(0.03 * len(got)))
-    assert len(bad) <= allowed, bad[:5]
+        assert err <= tol, (rid, p, float(err))
+
+
+CLOSE_CALL = 0.06      # (the expert block alone, bfloat16: routing choices made by less than this are left out)
 
 
 DEVICES = [pytest.param("cpu", "float32", 2e-4, id="cpu-f32"),
@@ -180,7 +191,7 @@ DEVICES = [pytest.param("cpu", "float32", 2e-4, id="cpu-f32"),
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_whole_prompt_and_first_tokens(name, device, dtype, tol, tmp_path_factory, tmp_path):
-    path, cfg, w = model_dir(name, tmp_path_factory)
+    path, cfg, w = model_dir(name, tmp_path_factory, dtype)
     reqs = {"a": tokens_for(cfg, 90, 1), "b": tokens_for(cfg, 1, 2), "c": tokens_for(cfg, 2, 3)}
     steps = [[(r, t, list(range(len(t)))), {"end": [r]}] for r, t in reqs.items()]
     got = run_schedule(path, steps, dtype, device, max_tokens=128, tmp=tmp_path)
@@ -195,7 +206,7 @@ def test_residual_stream_after_every_layer(device, dtype, tol, tmp_path_factory)
         pytest.skip("the per-layer comparison is the float32 one")
     from vllm_distributed_amd.entrypoints import trace_replay
     import types
-    path, cfg, w = model_dir("varied", tmp_path_factory)
+    path, cfg, w = model_dir("varied", tmp_path_factory, dtype)
     toks = tokens_for(cfg, 37, 8)
     args = types.SimpleNamespace(model=path, dtype=dtype, out="", max_tokens=64, max_seqs=2, device=device,
                                  block_size=16, enforce_eager=True)
@@ -218,11 +229,11 @@ def test_residual_stream_after_every_layer(device, dtype, tol, tmp_path_factory)
 
 
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
-@pytest.mark.parametrize("name", ["varied", "paged", "recurrent_only"])
+@pytest.mark.parametrize("name", ["varied", "paged", "recurrent_only", "fragments"])
 def test_prefill_then_long_token_by_token_decoding(name, device, dtype, tol, tmp_path_factory, tmp_path):
     """A prompt, then 150 tokens one at a time: the state is carried through 150 single-row steps, the cache grows
     over several pages."""
-    path, cfg, w = model_dir(name, tmp_path_factory)
+    path, cfg, w = model_dir(name, tmp_path_factory, dtype)
     toks = tokens_for(cfg, 190, 4)
     got = run_schedule(path, portions(toks, [40, 1], "r"), dtype, device, max_tokens=192, tmp=tmp_path)
     assert len(got) == 190
@@ -232,7 +243,7 @@ def test_prefill_then_long_token_by_token_decoding(name, device, dtype, tol, tmp
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
 @pytest.mark.parametrize("sizes", [[2], [3, 2, 7, 1, 16, 17, 2, 2, 31, 5], [1], [64, 2, 1]])
 def test_portions_of_any_size(sizes, device, dtype, tol, tmp_path_factory, tmp_path):
-    path, cfg, w = model_dir("varied", tmp_path_factory)
+    path, cfg, w = model_dir("varied", tmp_path_factory, dtype)
     toks = tokens_for(cfg, 75 if sizes != [1] else 40, 5)
     got = run_schedule(path, portions(toks, sizes, "r"), dtype, device, max_tokens=128, tmp=tmp_path)
     assert len(got) == len(toks)
@@ -247,7 +258,7 @@ def test_mixed_batches_reuse_pages_and_slots(device, dtype, tol, eager, tmp_path
     what the old one left); every row against the request run alone by the oracle."""
     if eager and device == "cpu":
         pytest.skip("graphs exist on the GPU only")
-    path, cfg, w = model_dir("paged", tmp_path_factory)
+    path, cfg, w = model_dir("paged", tmp_path_factory, dtype)
     reqs = {f"q{i}": tokens_for(cfg, n, 10 + i) for i, n in enumerate([50, 33, 1, 47, 20, 48, 9])}
     at = {r: 0 for r in reqs}
     pattern = {"q0": [7, 1, 1, 2, 30, 1], "q1": [2, 16, 1, 1, 1], "q2": [1], "q3": [17, 1, 15, 1], "q4": [1, 1, 5],
@@ -279,7 +290,7 @@ def test_mixed_batches_reuse_pages_and_slots(device, dtype, tol, eager, tmp_path
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
 def test_batch_rows_equal_single_runs(device, dtype, tol, tmp_path_factory, tmp_path):
     """The same rows run alone and inside a batch of unequal neighbours agree far inside the oracle tolerance."""
-    path, cfg, w = model_dir("varied", tmp_path_factory)
+    path, cfg, w = model_dir("varied", tmp_path_factory, dtype)
     a, b, c = tokens_for(cfg, 30, 20), tokens_for(cfg, 11, 21), tokens_for(cfg, 64, 22)
     alone = run_schedule(path, portions(a, [13, 1], "a"), dtype, device, max_tokens=64, tmp=tmp_path / "x")
     steps = [[("c", c[:50], []), ("a", a[:13], list(range(13))), ("b", b[:2], [])]]
@@ -392,13 +403,14 @@ def test_routing_rules(device):
         assert (w2.cpu().gather(1, i2.long().cpu().argsort(-1)).double() - wts.gather(1, idx.argsort(-1))).abs().max().item() < 1e-5
 
 
+@pytest.mark.parametrize("hidden", [40, 48])
 @pytest.mark.parametrize("device,dtype", OP_DEVICES)
-def test_expert_block_against_the_oracle(device, dtype):
+def test_expert_block_against_the_oracle(device, dtype, hidden):
     """The whole block - router, clamped experts with inputs beyond the limit, identity share, gated shared expert -
     on sizes that are no multiple of anything."""
     from vllm_distributed_amd.models.layers.moe import GroupedIdentityMoE
     dt = getattr(torch, dtype)
-    hidden, ff, experts, identity, top = 40, 24, 5, 1, 3
+    ff, experts, identity, top = 24, 5, 1, 3
     mlp = {"expert": {"ff": ff, "limit": 0.6}, "router": {"experts": experts, "identity": identity, "top": top,
                                                          "groups": {"count": 3, "keep": 2}}, "shared": {"ff": 16, "limit": 0.9}}
     g = torch.Generator().manual_seed(2)
@@ -423,11 +435,14 @@ def test_expert_block_against_the_oracle(device, dtype):
     m.shared.w2.data.copy_(w["shared.down"])
     m.shared_gate.weight.data.copy_(w["shared.sg"])
     x = (torch.randn(50, hidden, generator=g) * 1.5).to(dt)
-    want = oracle.moe(x.double(), {"p." + k: v for k, v in w.items()}, "p.", mlp)
+    margins = []
+    want = oracle.moe(x.double(), {"p." + k: v for k, v in w.items()}, "p.", mlp, margins)
     got = m(x.to(device)).cpu().double()
     err = (got - want).abs().max(-1).values
-    tol = 1e-4 if dtype == "float32" else 0.08
-    assert (err > tol).sum().item() <= (0 if dtype == "float32" else 2), err.max().item()
+    if dtype != "float32":
+        err = err[margins[0] >= CLOSE_CALL]
+        assert len(err) > 20
+    assert err.max().item() <= (1e-4 if dtype == "float32" else 0.08), err.max().item()
 
 
 def test_rotary_frequencies_and_partial_rotation():
@@ -545,7 +560,7 @@ def test_greedy_generation_through_the_scheduler(device, dtype, tmp_path_factory
     chunking and sampling.  Every generated token is the oracle's argmax given the tokens before it (in bfloat16: or
     its logit is within rounding of the oracle's best)."""
     from vllm_distributed_amd import LLM, SamplingParams
-    path, cfg, w = model_dir("varied", tmp_path_factory)
+    path, cfg, w = model_dir("varied", tmp_path_factory, dtype)
     prompts = [tokens_for(cfg, n, 40 + n) for n in (3, 30, 1, 17, 45)]
     llm = LLM(model=path, device=device, dtype=dtype, max_model_len=128, max_num_seqs=2, max_num_batched_tokens=16,
               block_size=16, load_format="safetensors", enforce_eager=False)

@@ -168,3 +168,36 @@ def test_latent_attention_decode_rows_and_one_far_key(dtype):
     lens0 = torch.tensor([0, 1, 0], dtype=torch.int32, device="cuda")
     o = hip.latent_row_attention(q, cache, table, None, lens0, 1.0, rank)
     assert torch.isfinite(o.float()).all() and o[0].float().abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("heads,rank,rope", [(6, 64, 32), (16, 512, 64), (20, 256, 64)])
+def test_fragment_cache_and_precise_matrix_core_attention(heads, rank, rope):
+    """Widths the matrix-core latent kernel is built for: ``latent_prep`` also writes the V^T fragments, and the
+    kernel with fp32-precise softmax weights agrees with the fp32 reference more closely than 8-bit weights could."""
+    hip = _hip()
+    from vllm_distributed_amd import ops
+    dtype = torch.bfloat16
+    c = _latent_case(dtype, heads, rank, rope, rope // 2, [(0, 1), (40, 1), (0, 33), (17, 20), (200, 4)], seed=rank)
+    nb, bs = c["cache"].shape[0], c["cache"].shape[2]
+    k1, k2 = c["cache"].clone(), c["cache"].clone()
+    v1 = torch.zeros(ops.v_cache_shape(nb, 1, rank, bs), dtype=dtype, device="cuda")
+    # the fragments of what is already cached
+    old = c["cache"][:, 0, :, :rank]                                            # [blocks, bs, rank]
+    v1[:, 0] = old.reshape(nb, bs // 8, 8, rank // 16, 16).permute(0, 3, 1, 4, 2)
+    v2 = v1.clone()
+    q1 = hip.latent_prep(c["q"], c["nope"], c["q_lat"], c["latent"], c["norm_w"], 1e-5, c["freq"], c["rs"], c["pos"], k1, c["slot"], v1)
+    q2 = torch_ref.latent_prep(c["q"], c["nope"], c["q_lat"], c["latent"], c["norm_w"], 1e-5, c["freq"], c["rs"], c["pos"], k2, c["slot"], v2)
+    _close(q1, q2, dtype, 8)
+    _close(k1, k2, dtype, 8)
+    _close(v1, v2, dtype, 8)
+    assert torch.equal(v2[:, 0].permute(0, 2, 4, 1, 3).reshape(nb, bs, rank), k2[:, 0, :, :rank])
+    qs = (q2.float() * 3).to(dtype)                                             # peaky softmax: weights near 1 matter
+    want = torch_ref.latent_row_attention(qs.float(), k2.float(), c["table"], c["rows"], c["lens"], 0.21, rank)
+    fine = hip.mla_attention(qs, k2, v2, c["table"], c["rows"], c["lens"], 0.21, 256, precise=True).float()
+    coarse = hip.mla_attention(qs, k2, v2, c["table"], c["rows"], c["lens"], 0.21, 256).float()
+    e_fine, e_coarse = (fine - want).abs().max().item(), (coarse - want).abs().max().item()
+    assert e_fine <= 6e-3 * max(1.0, want.abs().max().item()), (e_fine, e_coarse)      # (the output's own 8 bits)
+    assert e_fine <= e_coarse + 1e-6
+    dec = hip.mla_attention(qs[:2], k2, v2, c["table"], None, torch.tensor([1, 41], dtype=torch.int32, device="cuda"),
+                            0.21, 64, precise=True).float()
+    _close(dec, want[:2], dtype, 1)

@@ -26,7 +26,6 @@ state is not sharded).
 """
 from __future__ import annotations
 
-import math
 from typing import Dict, Iterable, List, Optional, Tuple
 
 import torch
@@ -88,7 +87,7 @@ class LatentMixer(nn.Module):
         self.uk = nn.Parameter(torch.empty(self.heads * self.nope, self.rank, dtype=dtype), requires_grad=False)
         self.uv = nn.Parameter(torch.empty(self.heads * self.vdim, self.rank, dtype=dtype), requires_grad=False)
         self.attn = RowLatentAttention(self.heads, self.rank, self.rope, float(m["scale"]), layer_idx,
-                                       source=None if source is None else source.attn)
+                                       source=None if source is None else source.attn, dtype=dtype)
         self.o = RowParallelLinear(self.heads * self.vdim, width, False, dtype)
         self._folded = None
 

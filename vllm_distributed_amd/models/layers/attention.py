@@ -253,9 +253,16 @@ class RowLatentAttention(Attention):
     row_cache = True
 
     def __init__(self, num_heads: int, rank: int, rope: int, scale: float, layer_idx: int,
-                 source: Optional["RowLatentAttention"] = None):
+                 source: Optional["RowLatentAttention"] = None, dtype: Optional[torch.dtype] = None):
         super().__init__(num_heads, rank + rope, 1, scale, layer_idx)
         self.rank, self.rope, self.v_dim = rank, rope, rank
+        # where the matrix-core latent kernel is built for this width and type, the values are cached once more as
+        # its V^T fragments and it serves the layer (with fp32-precise softmax weights); else the plain kernel
+        on_gpu = torch.empty(0).device.type != "cpu"       # (modules are built under the target device)
+        self.fragments = bool(on_gpu and dtype is not None and rank % 16 == 0
+                              and ops.mla_kernel_ok(rank + rope, rank, dtype))
+        if source is not None:
+            self.fragments = source.fragments
         if source is not None and (source.rank, source.rope) != (rank, rope):
             raise ValueError(f"layer {layer_idx} reads the latent rows of layer {source.layer_idx}, which have "
                              f"another shape ({source.rank} + {source.rope} against {rank} + {rope})")
@@ -263,10 +270,12 @@ class RowLatentAttention(Attention):
         object.__setattr__(self, "source", source)
 
     def kv_cache_shapes(self, num_blocks: int, block_size: int):
+        if self.fragments:
+            return (num_blocks, 1, block_size, self.head_dim), ops.v_cache_shape(num_blocks, 1, self.rank, block_size)
         return (num_blocks, 1, block_size, self.head_dim), (num_blocks, 0)
 
     def kv_values_per_token(self) -> int:
-        return self.head_dim
+        return self.head_dim + (self.rank if self.fragments else 0)
 
     def bind_kv_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_scales: Optional[tuple] = None) -> None:
         if k_cache.dtype == torch.float8_e4m3fn:
@@ -286,10 +295,15 @@ class RowLatentAttention(Attention):
         md, pos = _CTX.attn_metadata, _CTX.positions
         write = latent is not None and self.source is None and md is not None
         qf = ops.latent_prep(q, nope, q_lat, latent if write else None, norm_weight, eps, inv_freq, rot_scale, pos,
-                             self.k_cache if write else None, md.slot_mapping if write else None)
+                             self.k_cache if write else None, md.slot_mapping if write else None,
+                             self.v_cache if write and self.fragments else None)
         if md is None:                          # memory-profiling pass: no cache bound
             return qf[..., :self.rank].contiguous()
         rows, lens = md.token_rows(pos)
+        if self.fragments:
+            owner = self.source if self.source is not None else self
+            return ops.mla_attention(qf, owner.k_cache, owner.v_cache, md.block_table, rows, lens, self.scale,
+                                     md.max_seq_len, precise=True)
         return ops.latent_row_attention(qf, self.rows, md.block_table, rows, lens, self.scale, self.rank, md.max_seq_len)
 
 

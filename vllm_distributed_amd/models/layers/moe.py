@@ -454,7 +454,8 @@ class GroupedIdentityMoE(FusedMoE):
         return F.linear(ops.clamped_glu(h, self.limit, self.alpha), self.w2[e])
 
     def _grouped_tile_rows(self, x: torch.Tensor) -> int:
-        if self.num_experts > 512 or self.top_k > 16 or self.groups > 64 or x.dim() != 2 or self.hidden % 8:
+        # (the grouped GEMMs write whole 16-column tiles: the down projection's output width is `hidden`)
+        if self.num_experts > 512 or self.top_k > 16 or self.groups > 64 or x.dim() != 2 or self.hidden % 16:
             return 0
         return super()._grouped_tile_rows(x)
 
@@ -465,7 +466,8 @@ class GroupedIdentityMoE(FusedMoE):
 
     def decode_capturable(self, dtype: torch.dtype) -> bool:
         """Whether a decode step of this block runs without a host synchronisation (the grouped path)."""
-        return dtype in (torch.bfloat16, torch.float16) and self.hidden % 8 == 0 and self.num_experts <= 512
+        return (dtype in (torch.bfloat16, torch.float16) and self.hidden % 16 == 0 and self.num_experts <= 512
+                and self.top_k <= 16 and self.groups <= 64)
 
     def _forward_routed(self, x: torch.Tensor) -> torch.Tensor:
         logits = self.router_logits(x)

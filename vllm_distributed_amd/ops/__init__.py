@@ -599,11 +599,14 @@ def mla_cache_write(latent, k_cache, v_cache, slot_mapping):
     return torch_ref.mla_cache_write(latent, k_cache, v_cache, slot_mapping)
 
 
-def mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out=None):
+def mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out=None,
+                  precise: bool = False):
+    """``precise``: softmax weights with fp32 precision in the weighted sum (models that define them in 32-bit)."""
     on_hip = _use_hip(q) and _hip.mla_supported(q.shape[2], v_cache.shape[2] * v_cache.shape[4], q.dtype)
     _note_attention(q, on_hip)
     if on_hip:
-        return _hip.mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out)
+        return _hip.mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out,
+                                  precise=precise)
     return torch_ref.mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out)
 
 
@@ -731,12 +734,12 @@ def relu_squared(x):
 
 
 def latent_prep(q, nope: int, q_lat, latent, norm_weight, eps: float, inv_freq, rot_scale: float, positions, cache,
-                slot_mapping):
+                slot_mapping, fragments=None):
     if _use_hip(q):
         return _hip.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
-                                slot_mapping)
+                                slot_mapping, fragments)
     return torch_ref.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
-                                 slot_mapping)
+                                 slot_mapping, fragments)
 
 
 def latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale: float, rank: int, max_seq_len: int = 0):

@@ -57,7 +57,7 @@ def load() -> ctypes.CDLL:
         "vdamd_moe_combine": [P, L, P, L, P, P, P, I, I, I, I, I, P, I, P],
         "vdamd_bias_clamped_glu": [P, L, P, L, P, P, P, I, I, I, I, F, F, I, P],
         "vdamd_moe_topk_grouped": [P, L, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
-        "vdamd_mla_attention": [P, L, P, P, P, L, P, P, P, I, P, P, F, I, I, I, I, I, I, I, I, I, P],
+        "vdamd_mla_attention": [P, L, P, P, P, L, P, P, P, I, P, P, F, I, I, I, I, I, I, I, I, I, I, P],
         "vdamd_mla_cache_write": [P, L, P, P, P, I, I, I, I, I, I, P],
         "vdamd_mla_prep": [P, P, L, I, I, P, L, L, P, L, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "vdamd_moe_combine_add_rms_norm": [P, L, P, L, P, P, P, I, I, I, I, I, P, P, F, I, P],
@@ -76,7 +76,7 @@ def load() -> ctypes.CDLL:
         "vdamd_clamped_glu": [P, P, L, I, I, F, F, I, P],
         "vdamd_relu_squared": [P, P, L, I, P],
         "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, P],
-        "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, I, I, I, I, I, P],
+        "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P],
     }
     for name, argtypes in sigs.items():
@@ -1150,12 +1150,13 @@ def mla_num_splits(tokens: int, q_tiles: int, max_seq_len: int) -> int:
 def mla_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                   token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, max_seq_len: int,
                   out: Optional[torch.Tensor] = None, splits: Optional[int] = None,
-                  mode: Optional[int] = None) -> torch.Tensor:
+                  mode: Optional[int] = None, precise: bool = False) -> torch.Tensor:
     """``q[T, Hq, DK]`` against the latent cache -> ``[T, Hq, DV]``; token ``t`` reads block-table row
     ``token_seq[t]`` (``t`` itself when None) and sees keys ``0 .. seq_lens[t] - 1``.  ``mode`` (default: by
     shape): 0 = a workgroup per (token, 16 heads); 1 = four consecutive tokens of a sequence per workgroup
     (steps with ``token_seq``: prefill chunks, verification - the tokens of a sequence must be adjacent rows at
-    consecutive positions); 2 = four head tiles of a token per workgroup (64 heads per rank and more)."""
+    consecutive positions); 2 = four head tiles of a token per workgroup (64 heads per rank and more).
+    ``precise``: the softmax weights enter the PV product with fp32 precision (a high and a low 16-bit part)."""
     t, hq, dk = q.shape
     dv = v_cache.shape[2] * v_cache.shape[4]
     bs = k_cache.shape[2]
@@ -1182,7 +1183,7 @@ def mla_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
         None if part_ml is None else part_ml.data_ptr(), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
         v_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         None if token_seq is None else token_seq.data_ptr(), seq_lens.data_ptr(), float(scale), t, hq, dk, dv, bs,
-        splits, int(mode), _dt(q), _mla_fp8(k_cache, v_cache, q.dtype), _stream()), "mla_attention")
+        splits, int(mode), _dt(q), _mla_fp8(k_cache, v_cache, q.dtype), int(bool(precise)), _stream()), "mla_attention")
     return out
 
 
@@ -1450,7 +1451,10 @@ def relu_squared(x: torch.Tensor) -> torch.Tensor:
 
 def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
                 norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
-                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> torch.Tensor:
+                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+                fragments: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``fragments``: the V^T fragment cache ``[blocks, 1, rank / 16, block / 8, 16, 8]`` of the matrix-core latent
+    attention kernel, written beside the rows when the layer keeps one."""
     t, h, qd = q.shape
     rank, rope = q_lat.shape[2], qd - nope
     half = inv_freq.numel()
@@ -1463,12 +1467,21 @@ def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optiona
         assert latent.shape == (t, rank + rope) and latent.stride(1) == 1 and latent.dtype == q.dtype
         assert cache.is_contiguous() and cache.dtype == q.dtype and cache.shape[1] == 1 and cache.shape[3] == rank + rope
         assert slot_mapping.dtype == torch.int32 and slot_mapping.numel() >= t
+        if fragments is not None and fragments.numel():
+            bs = cache.shape[2]
+            assert fragments.is_contiguous() and fragments.dtype == q.dtype and rank % 16 == 0 and bs % 8 == 0
+            assert tuple(fragments.shape[1:]) == (1, rank // 16, bs // 8, 16, 8) and fragments.shape[0] == cache.shape[0]
+        else:
+            fragments = None
+    else:
+        fragments = None
     _check(_LIB.vdamd_latent_prep(
         out.data_ptr(), q.data_ptr(), q.stride(0), q.stride(1), nope, q_lat.data_ptr(), q_lat.stride(0),
         q_lat.stride(1), latent.data_ptr() if write else None, latent.stride(0) if write else 0,
         _f32_vec(norm_weight, rank, "norm_weight").data_ptr() if write else None, float(eps), inv_freq.data_ptr(),
-        half, float(rot_scale), positions.data_ptr(), cache.data_ptr() if write else None,
-        slot_mapping.data_ptr() if write else None, t, h, rank, rope, _dt(q), _stream()), "latent_prep")
+        half, float(rot_scale), positions.data_ptr(), cache.data_ptr() if write else None, _ptr(fragments),
+        slot_mapping.data_ptr() if write else None, t, h, rank, rope, cache.shape[2] if write else 8, _dt(q),
+        _stream()), "latent_prep")
     return out
 
 

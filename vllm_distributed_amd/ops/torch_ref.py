@@ -670,13 +670,15 @@ def rotate_half_first(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.
 
 def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
                 norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
-                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> torch.Tensor:
+                positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+                fragments: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Between the projections and the attention of a layer whose keys and values are one shared latent row per
     token.  ``q[T, H, nope + rope]``, ``q_lat[H, T, rank]`` (the unrotated query part already multiplied into the
     latent space): returns ``[T, H, rank + rope] = [q_lat | rotated q[..., nope:]]``.  With ``latent[T, rank + rope]``
     the row ``[RMS norm of the first rank values * norm_weight | rotated last rope values]`` goes into
     ``cache[blocks, 1, block, rank + rope]`` at ``slot_mapping`` (a layer that reads another layer's rows passes
-    None).  Norm and rotation in fp32."""
+    None), and its first ``rank`` values also into ``fragments`` (the V^T fragment cache, see ``v_cache_shape``) when
+    the layer keeps one.  Norm and rotation in fp32."""
     t = q.shape[0]
     q_rot = rotate_half_first(q[..., nope:].float(), positions[:t], inv_freq, rot_scale)
     out = torch.cat([q_lat.transpose(0, 1).float(), q_rot], dim=-1).to(q.dtype)
@@ -690,6 +692,9 @@ def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optiona
         valid = slot_mapping[:t] >= 0
         sm = slot_mapping[:t][valid].long()
         cache[sm // bs, 0, sm % bs, :] = row[valid]
+        if fragments is not None and fragments.numel():       # the values once more, as V^T fragments
+            off = sm % bs
+            fragments[sm // bs, 0, :, off // V_GROUP, :, off % V_GROUP] = row[valid][:, :rank].unflatten(-1, (-1, V_ROWS))
     return out
 
 
