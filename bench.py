@@ -139,11 +139,14 @@ def _parse():
     ap.add_argument("--alt-parallelism", type=str, default="pp",
                     help="second layout measured in a child process after the headline when N > 1 ('none' = skip)")
     ap.add_argument("--alt-timeout", type=float, default=900.0)
-    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix"],
+    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix", "kabapel"],
                     help="instead of the headline: prefill and decode throughput of this model family at a few layer "
-                         "sizes beside the closest existing family (Gemma-2) at equal size, random weights, one GPU")
+                         "sizes beside the closest existing family at equal size (Tavulix: Gemma-2; Kabapel: "
+                         "DeepSeek-V2), random weights, one GPU")
     ap.add_argument("--compare-sizes", type=str, default="small,medium",
                     help="with --family-compare: which of small / medium / large to run")
+    ap.add_argument("--compare-only", type=str, default=None,
+                    help="with --family-compare: run just this one of the two families (for a kernel trace of it)")
     ap.add_argument("--device", type=str, default="cuda", choices=["cuda", "cpu"],
                     help="cpu = gloo rehearsal of the multi-rank path with a tiny model (not a measurement)")
     return ap.parse_args()
@@ -223,6 +226,54 @@ def _compare_models(z: dict) -> dict:
     return {"tavulix": ("tavulix-tiny", tav), "gemma2": ("gemma2-tiny", gem)}
 
 
+KABAPEL_SIZES = {
+    "tiny": dict(width=128, heads=4, rank=64, rope=32, nope=32, vdim=32, experts=6, identity=2, top=2, groups=(4, 2), ff=64,
+                 shared=128, layers=4, prompt=96, prompts=2, batch=4),
+    # width, heads, latent rank, rotated / unrotated key part, value size, experts (+ identity outputs), chosen, groups
+    # (count, kept), expert and shared feed-forward, layers, prompt length, prefill prompts, decode batch
+    "small": dict(width=1024, heads=8, rank=512, rope=64, nope=128, vdim=128, experts=14, identity=2, top=4, groups=(4, 2),
+                  ff=512, shared=1024, layers=4, prompt=1024, prompts=16, batch=64),
+    "medium": dict(width=2048, heads=16, rank=512, rope=64, nope=128, vdim=128, experts=30, identity=2, top=4, groups=(8, 4),
+                   ff=1024, shared=2048, layers=4, prompt=2048, prompts=8, batch=128),
+    "large": dict(width=4096, heads=32, rank=512, rope=64, nope=128, vdim=128, experts=62, identity=2, top=6, groups=(8, 4),
+                  ff=1408, shared=2816, layers=2, prompt=4096, prompts=4, batch=128),
+}
+
+
+def _kabapel_models(z: dict) -> dict:
+    """The same layer sizes as a Kabapel config (recurrent and latent layers in turn, the second latent layer reading
+    the first one's rows) and as a DeepSeek-V2 config (latent attention, grouped routing, shared experts: the closest
+    family the framework has)."""
+    vocab = 32000
+    rot = {"base": 10000.0, "dims": z["rope"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"],
+                      "groups": {"count": z["groups"][0], "keep": z["groups"][1]}},
+           "shared": {"ff": z["shared"], "limit": 7.0}}
+    lat = {"heads": z["heads"], "dim": z["nope"], "rot_dim": z["rope"], "vdim": z["vdim"], "kv_rank": z["rank"],
+           "scale": (z["nope"] + z["rope"]) ** -0.5, "rot": rot}
+    lin = {"heads": z["heads"], "dim": z["nope"], "vdim": z["vdim"],
+           "decay": [1.0 - 2.0 ** -(2 + 6 * h / max(z["heads"] - 1, 1)) for h in range(z["heads"])]}
+    layers, first_latent = [], None
+    for i in range(z["layers"]):
+        if i % 2 == 0:
+            layers.append({"type": "lightning", "mixer": lin, "mlp": moe})
+        else:
+            m = dict(lat) if first_latent is None else dict(lat, kv_from=first_latent)
+            first_latent = i if first_latent is None else first_latent
+            layers.append({"type": "latent_attention", "mixer": m, "mlp": moe})
+    kab = {"architecture": "Kabapel", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-5},
+           "embedding": {"scale": 1.0}, "layers": layers}
+    dsk = {"hidden_size": z["width"], "num_attention_heads": z["heads"], "num_key_value_heads": z["heads"],
+           "kv_lora_rank": z["rank"], "qk_nope_head_dim": z["nope"], "qk_rope_head_dim": z["rope"], "v_head_dim": z["vdim"],
+           "q_lora_rank": None, "n_routed_experts": z["experts"] + z["identity"], "num_experts_per_tok": z["top"],
+           "moe_intermediate_size": z["ff"], "n_shared_experts": max(z["shared"] // z["ff"], 1),
+           "n_group": z["groups"][0], "topk_group": z["groups"][1], "topk_method": "group_limited_greedy",
+           "first_k_dense_replace": 0, "num_hidden_layers": z["layers"], "vocab_size": vocab,
+           "max_position_embeddings": 8192, "rope_scaling": None, "torch_dtype": "bfloat16"}
+    return {"kabapel": ("kabapel-tiny", kab), "deepseek_v2": ("deepseek-v2-lite", dsk)}
+
+
 def run_family_compare(args) -> None:
     """Prefill throughput (``prompts`` prompts of ``prompt`` tokens, one generated token each) and decode
     throughput (``batch`` sequences, 64 further tokens each; the prefill time measured the same way is taken off)
@@ -232,9 +283,12 @@ def run_family_compare(args) -> None:
     from vllm_distributed_amd import LLM, SamplingParams
     os.environ.setdefault("VLLM_LOGGING_LEVEL", "WARNING")
     rows = []
+    kabapel = args.family_compare == "kabapel"
     for size in [s for s in args.compare_sizes.split(",") if s]:
-        z = COMPARE_SIZES[size]
-        for family, (base, over) in _compare_models(z).items():
+        z = (KABAPEL_SIZES if kabapel else COMPARE_SIZES)[size]
+        for family, (base, over) in (_kabapel_models(z) if kabapel else _compare_models(z)).items():
+            if args.compare_only and family != args.compare_only:
+                continue
             llm = LLM(model=base, hf_overrides=over, dtype=args.dtype, device=args.device, load_format="dummy",
                       max_model_len=z["prompt"] + 128, max_num_seqs=max(z["batch"], z["prompts"]),
                       max_num_batched_tokens=8192, gpu_memory_utilization=0.5, enforce_eager=args.enforce_eager,

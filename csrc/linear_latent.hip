@@ -12,6 +12,7 @@
 //   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g)
 //   clamped_glu              min(g, L) sigmoid(alpha min(g, L)) (clamp(u, -L, L) + 1) over [g | u]
 //   relu_squared             max(x, 0)^2
+//   expert_epilogue          routed + x * (weights of the chosen identity experts) + shared * sigmoid(gate)
 //   latent_prep              per token: RMS norm of the latent and rotation of the shared key part into the row cache;
 //                            the query [q_lat | rotated q_rope] assembled; angles = position * frequency in fp32
 //   latent_row_attention     causal softmax attention of every head over the shared rows (value = a row's first
@@ -109,6 +110,63 @@ __global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ h,
   }
 }
 
+// 16-bit rows whose length and stride are multiples of 8: 16-byte accesses
+template <typename T>
+__global__ void clamped_glu_vec_kernel(T* __restrict__ out, const T* __restrict__ h, long h_stride, int F, float limit,
+                                       float alpha) {
+  using V8 = typename Vec8<T>::type;
+  const long row = blockIdx.x;
+  const T* hr = h + row * h_stride;
+  T* o = out + row * (long)F;
+  for (int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8; i < F; i += gridDim.y * blockDim.x * 8) {
+    const V8 gv = ld8<T>(hr + i), uv = ld8<T>(hr + F + i);
+    V8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float g = fminf((float)gv[e], limit);
+      const float u = fminf(fmaxf((float)uv[e], -limit), limit);
+      r[e] = (T)(g * sigmoid_f(alpha * g) * (u + 1.0f));
+    }
+    st8<T>(o + i, r);
+  }
+}
+
+// out = routed + x * (sum of the weights of the chosen outputs that are identity experts) + shared * sigmoid(gate):
+// what follows the routed experts of a block with identity experts and a gated shared expert, in one pass
+template <typename T>
+__global__ void expert_epilogue_kernel(T* __restrict__ out, const T* __restrict__ routed, const T* __restrict__ x,
+                                       long x_stride, const float* __restrict__ topw, const int* __restrict__ topi,
+                                       int k, int real_experts, const T* __restrict__ shared,
+                                       const T* __restrict__ gate, long gate_stride, int H) {
+  const long row = blockIdx.x;
+  float share = 0.f;
+  if (topw != nullptr)
+    for (int j = 0; j < k; ++j)
+      if (topi[row * k + j] >= real_experts) share += topw[row * k + j];
+  const float g = gate != nullptr ? sigmoid_f(ldf(gate + row * gate_stride)) : 0.f;
+  const T* rr = routed + row * (long)H;
+  const T* xr = x + row * x_stride;
+  const T* sr = shared != nullptr ? shared + row * (long)H : nullptr;
+  T* o = out + row * (long)H;
+  if constexpr (!std::is_same_v<T, float>) {
+    if ((H & 7) == 0 && (x_stride & 7) == 0) {
+      using V8 = typename Vec8<T>::type;
+      for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+        const V8 rv = ld8<T>(rr + i), xv = ld8<T>(xr + i);
+        V8 sv = rv, res;
+        if (sr != nullptr) sv = ld8<T>(sr + i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          res[e] = (T)((float)rv[e] + (float)xv[e] * share + (sr != nullptr ? (float)sv[e] * g : 0.f));
+        st8<T>(o + i, res);
+      }
+      return;
+    }
+  }
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    stf(o + i, ldf(rr + i) + ldf(xr + i) * share + (sr != nullptr ? ldf(sr + i) * g : 0.f));
+}
+
 template <typename T>
 __global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ x, long n) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
@@ -119,19 +177,29 @@ __global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ x
 
 // ------------------------------------------------------------------------------------------------ linear attention
 // grid (sequences, heads, column tiles of 64), 256 threads: thread (g = tid / 64, c = tid % 64) owns rows
-// g * R .. g * R + R - 1 of column c of the head's state.  x rows hold [q (H * dim) | k (H * dim) | v (H * vdim) | ..].
-// One barrier per row: q / k of the row are staged in LDS (double-buffered), the four row groups' partial outputs of
-// the previous row are summed after the next barrier.
+// g * R .. g * R + R - 1 of column c of the head's state, in registers.  x rows hold [q (H * dim) | k (H * dim) |
+// v (H * vdim) | ..].  The sequence's rows are walked in chunks of DLA_CHUNK: q / k (all of the head) and v (this
+// tile's columns) of a chunk are staged in LDS through SiLU, the next chunk's loads are in flight while the current
+// one is computed, and the four row groups' partial outputs of a chunk are summed after one barrier - two barriers
+// per chunk whatever its length, so a single decoded row and a long prompt portion are the same launch.
+constexpr int DLA_CHUNK = 16;
+
 template <typename T, int R>
 __global__ __launch_bounds__(256) void decay_linear_attention_kernel(
     float* __restrict__ out, const T* __restrict__ x, long x_stride, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int H, int dim, int vdim, int silu) {
-  __shared__ float qs[2][4 * R], ks[2][4 * R], part[2][4][64];
+  constexpr int C = DLA_CHUNK, W = 4 * R;          // W: the key size padded to the four row groups
+  constexpr int NQ = C * W / 256;                  // q (and k) values a thread stages per chunk
+  constexpr int NV = C * 64 / 256;
+  __shared__ __attribute__((aligned(16))) float qs[C][W];
+  __shared__ __attribute__((aligned(16))) float ks[C][W];
+  __shared__ float vs[C][64];
+  __shared__ float part[4][C][64];
   const int b = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, g = tid >> 6, lane = tid & 63;
-  const int c = blockIdx.z * 64 + lane;
-  const bool col = c < vdim;
+  const int col0 = blockIdx.z * 64;
+  const bool col = col0 + lane < vdim;
   const int s = qsl[b], e = qsl[b + 1];
   if (e <= s) return;                                            // (uniform over the workgroup)
   const int start = seq_lens[b] - (e - s);
@@ -141,50 +209,71 @@ __global__ __launch_bounds__(256) void decay_linear_attention_kernel(
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int r = g * R + i;
-    S[i] = (start > 0 && col && r < dim) ? st[(long)r * vdim + c] : 0.f;
+    S[i] = (start > 0 && col && r < dim) ? st[(long)r * vdim + col0 + lane] : 0.f;
   }
-  const long qoff = (long)h * dim, koff = (long)(H + h) * dim, voff = 2L * H * dim + (long)h * vdim + c;
+  const long qoff = (long)h * dim, koff = (long)(H + h) * dim, voff = 2L * H * dim + (long)h * vdim + col0;
   auto act = [&](float f) { return silu ? f * sigmoid_f(f) : f; };
-  // rows beyond `dim` of the staging buffers stay zero
-  for (int i = tid; i < 4 * R; i += 256) { qs[0][i] = qs[1][i] = ks[0][i] = ks[1][i] = 0.f; }
-  float nq = 0.f, nk = 0.f, nv = 0.f;
-  {
-    const T* xr = x + (long)s * x_stride;
-    if (tid < dim) { nq = act(ldf(xr + qoff + tid)); nk = act(ldf(xr + koff + tid)); }
-    if (col) nv = act(ldf(xr + voff));
-  }
-  __syncthreads();
-  for (int r = s; r < e; ++r) {
-    const int buf = (r - s) & 1;
-    if (tid < dim) { qs[buf][tid] = nq; ks[buf][tid] = nk; }
-    const float v = nv;
-    if (r + 1 < e) {
-      const T* xr = x + (long)(r + 1) * x_stride;
-      if (tid < dim) { nq = act(ldf(xr + qoff + tid)); nk = act(ldf(xr + koff + tid)); }
-      if (col) nv = act(ldf(xr + voff));
+  float pq[NQ], pk[NQ], pv[NV];
+  auto fetch = [&](int r0) {                       // rows r0 .. of the sequence into registers (zero beyond its end)
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int idx = tid + 256 * u, t = idx / W, j = idx - t * W;
+      const bool ok = r0 + t < e && j < dim;
+      const T* xr = x + (long)(r0 + t) * x_stride;
+      pq[u] = ok ? act(ldf(xr + qoff + j)) : 0.f;
+      pk[u] = ok ? act(ldf(xr + koff + j)) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + 256 * u, t = idx >> 6, c = idx & 63;
+      const bool ok = r0 + t < e && col0 + c < vdim;
+      pv[u] = ok ? act(ldf(x + (long)(r0 + t) * x_stride + voff + c)) : 0.f;
+    }
+  };
+  fetch(s);
+  for (int r0 = s; r0 < e; r0 += C) {
+    const int n = min(C, e - r0);
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int idx = tid + 256 * u, t = idx / W, j = idx - t * W;
+      qs[t][j] = pq[u];
+      ks[t][j] = pk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + 256 * u;
+      vs[idx >> 6][idx & 63] = pv[u];
+    }
+    if (r0 + C < e) fetch(r0 + C);
+    __syncthreads();
+    for (int t = 0; t < n; ++t) {
+      const float v = vs[t][lane];
+      const float4* k4 = reinterpret_cast<const float4*>(&ks[t][g * R]);
+      const float4* q4 = reinterpret_cast<const float4*>(&qs[t][g * R]);
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < R / 4; ++i) {
+        const float4 kk = k4[i], qq = q4[i];
+        S[4 * i] = d * S[4 * i] + kk.x * v;         acc += S[4 * i] * qq.x;
+        S[4 * i + 1] = d * S[4 * i + 1] + kk.y * v; acc += S[4 * i + 1] * qq.y;
+        S[4 * i + 2] = d * S[4 * i + 2] + kk.z * v; acc += S[4 * i + 2] * qq.z;
+        S[4 * i + 3] = d * S[4 * i + 3] + kk.w * v; acc += S[4 * i + 3] * qq.w;
+      }
+      part[g][t][lane] = acc;
     }
     __syncthreads();
-    if (r > s && g == 0 && col)
-      out[(long)(r - 1) * H * vdim + (long)h * vdim + c] =
-          (part[buf ^ 1][0][lane] + part[buf ^ 1][1][lane]) + (part[buf ^ 1][2][lane] + part[buf ^ 1][3][lane]);
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < R; ++i) {
-      S[i] = d * S[i] + ks[buf][g * R + i] * v;
-      acc += S[i] * qs[buf][g * R + i];
+    for (int idx = tid; idx < n * 64; idx += 256) {
+      const int t = idx >> 6, c = idx & 63;
+      if (col0 + c < vdim)
+        out[(long)(r0 + t) * H * vdim + (long)h * vdim + col0 + c] =
+            (part[0][t][c] + part[1][t][c]) + (part[2][t][c] + part[3][t][c]);
     }
-    part[buf][g][lane] = acc;
   }
-  __syncthreads();
-  const int last = (e - 1 - s) & 1;
-  if (g == 0 && col)
-    out[(long)(e - 1) * H * vdim + (long)h * vdim + c] =
-        (part[last][0][lane] + part[last][1][lane]) + (part[last][2][lane] + part[last][3][lane]);
   if (col) {
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const int r = g * R + i;
-      if (r < dim) st[(long)r * vdim + c] = S[i];
+      if (r < dim) st[(long)r * vdim + col0 + lane] = S[i];
     }
   }
 }
@@ -406,8 +495,33 @@ VDAMD_API int vdamd_clamped_glu(void* out, const void* h, long h_stride, int row
   if (F <= 0) return 1;
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
+    if constexpr (!std::is_same_v<TT, float>) {
+      if (F % 8 == 0 && h_stride % 8 == 0) {
+        hipLaunchKernelGGL((clamped_glu_vec_kernel<TT>), dim3(rows, (F + 2047) / 2048), dim3(256), 0, stream, (TT*)out,
+                           (const TT*)h, h_stride, F, limit, alpha);
+        return;
+      }
+    }
     hipLaunchKernelGGL((clamped_glu_kernel<TT>), dim3(rows, (F + 1023) / 1024), dim3(256), 0, stream, (TT*)out,
                        (const TT*)h, h_stride, F, limit, alpha);
+  });
+  if (rc) return 1;
+  HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+// routed, shared (may be null), out: [rows, H] contiguous; x rows x_stride apart; topw / topi [rows, k] (may be null:
+// no identity share); gate (may be null with shared) one value per row, gate_stride apart
+VDAMD_API int vdamd_expert_epilogue(void* out, const void* routed, const void* x, long x_stride, const float* topw,
+                                    const int* topi, int k, int real_experts, const void* shared, const void* gate,
+                                    long gate_stride, int rows, int H, int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || (topw != nullptr && (topi == nullptr || k < 1)) || (shared != nullptr && gate == nullptr)) return 1;
+  const int rc = by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    hipLaunchKernelGGL((expert_epilogue_kernel<TT>), dim3(rows), dim3(H >= 2048 ? 256 : 128), 0, stream, (TT*)out,
+                       (const TT*)routed, (const TT*)x, x_stride, topw, topi, k, real_experts, (const TT*)shared,
+                       (const TT*)gate, gate_stride, H);
   });
   if (rc) return 1;
   HIP_LAUNCH_CHECK();

@@ -201,3 +201,20 @@ def test_fragment_cache_and_precise_matrix_core_attention(heads, rank, rope):
     dec = hip.mla_attention(qs[:2], k2, v2, c["table"], None, torch.tensor([1, 41], dtype=torch.int32, device="cuda"),
                             0.21, 64, precise=True).float()
     _close(dec, want[:2], dtype, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("h", [40, 320, 2048])
+def test_expert_epilogue(dtype, h):
+    hip = _hip()
+    g = torch.Generator(device="cuda").manual_seed(h)
+    t, k = 9, 3
+    routed = torch.randn(t, h, device="cuda", generator=g).to(dtype)
+    x = torch.randn(t, h + 8, device="cuda", generator=g).to(dtype)[:, :h]
+    shared = torch.randn(t, h, device="cuda", generator=g).to(dtype)
+    gate = torch.randn(t, 1, device="cuda", generator=g).to(dtype)
+    topw = torch.rand(t, k, device="cuda", generator=g)
+    topi = torch.randint(0, 8, (t, k), device="cuda", generator=g).to(torch.int32)
+    for args in ((topw, topi, 5, shared, gate), (None, None, 5, shared, gate), (topw, topi, 5, None, None),
+                 (topw, topi, 8, shared, gate)):
+        _close(hip.expert_epilogue(routed, x, *args), torch_ref.expert_epilogue(routed, x, *args), dtype, 4)

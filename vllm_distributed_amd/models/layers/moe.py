@@ -402,9 +402,10 @@ class GroupedIdentityMoE(FusedMoE):
         self.local_experts, self.expert_start = num_experts, 0      # the identity outputs have no weights
         self.groups, self.keep_groups = groups, keep_groups
         self.limit, self.alpha = float(limit), float(alpha)
-        f32 = torch.float32
-        self.gate = ReplicatedLinear(hidden, outputs, False, f32, quant=False)
-        self.gate.e_score_correction_bias = nn.Parameter(torch.zeros(outputs, dtype=f32), requires_grad=False)
+        # (router weights in the model dtype: what a 16-bit checkpoint holds is exact there, and the product is
+        # formed with fp32 accumulators kept as the result)
+        self.gate = ReplicatedLinear(hidden, outputs, False, dtype, quant=False)
+        self.gate.e_score_correction_bias = nn.Parameter(torch.zeros(outputs, dtype=torch.float32), requires_grad=False)
         self.h_pad, self.i_pad = _ceil128(hidden), _ceil128(inter)
         E = num_experts
         # [gate rows ; up rows] (each padded to i_pad rows) x (reduction padded to h_pad); [hidden, i_pad]
@@ -430,7 +431,7 @@ class GroupedIdentityMoE(FusedMoE):
 
     # ------------------------------------------------------------------ routing
     def router_logits(self, x: torch.Tensor) -> torch.Tensor:
-        return F.linear(x.float(), self.gate.weight)
+        return ops.linear_f32(x, self.gate.weight)
 
     def route(self, logits: torch.Tensor):
         scores = torch.softmax(logits.float(), dim=-1)
@@ -459,17 +460,12 @@ class GroupedIdentityMoE(FusedMoE):
             return 0
         return super()._grouped_tile_rows(x)
 
-    def _identity_share(self, topw: torch.Tensor, topi: torch.Tensor) -> Optional[torch.Tensor]:
-        if not self.identity:
-            return None
-        return (topw * (topi >= self.real_experts)).sum(-1, keepdim=True)
-
     def decode_capturable(self, dtype: torch.dtype) -> bool:
         """Whether a decode step of this block runs without a host synchronisation (the grouped path)."""
         return (dtype in (torch.bfloat16, torch.float16) and self.hidden % 16 == 0 and self.num_experts <= 512
                 and self.top_k <= 16 and self.groups <= 64)
 
-    def _forward_routed(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, reduce: bool = True, staged: bool = False, deferred: bool = False):
         logits = self.router_logits(x)
         tile_rows = self._grouped_tile_rows(x)
         if tile_rows:
@@ -481,30 +477,26 @@ class GroupedIdentityMoE(FusedMoE):
             h = ops.grouped_linear(xs, tiles, tile_rows, weight=self.w13)
             y = ops.grouped_linear(ops.clamped_glu(h, self.limit, self.alpha), tiles, tile_rows, weight=self.w2)
             out = ops.moe_combine(y, topw, topi, inv, 0, self.real_experts)
-            share = self._identity_share(topw, topi.long())
-            return out if share is None else out + (x.float() * share).to(x.dtype)
-        topw, topi = self.route(logits)
-        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
-        flat_e = topi.reshape(-1)
-        order = flat_e.argsort(stable=True)
-        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()
-        tok = order // self.top_k
-        wts = topw.reshape(-1)[order]
-        start = 0
-        for eid, n in enumerate(counts[:self.real_experts]):
-            if n:
-                seg = slice(start, start + n)
-                rows = tok[seg]
-                out.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
-            start += n
-        share = self._identity_share(topw, topi)
-        if share is not None:
-            out += x.float() * share
-        return out.to(x.dtype)
-
-    def forward(self, x: torch.Tensor, reduce: bool = True, staged: bool = False, deferred: bool = False):
-        out = self._forward_routed(x)
+        else:
+            topw, topi = self.route(logits)
+            acc = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            flat_e = topi.reshape(-1)
+            order = flat_e.argsort(stable=True)
+            counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()
+            tok = order // self.top_k
+            wts = topw.reshape(-1)[order]
+            start = 0
+            for eid, n in enumerate(counts[:self.real_experts]):
+                if n:
+                    seg = slice(start, start + n)
+                    rows = tok[seg]
+                    acc.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
+                start += n
+            out = acc.to(x.dtype)
+        if not self.identity and self.shared is None:
+            return out
+        shared = gate = None
         if self.shared is not None:
-            g = torch.sigmoid(self.shared_gate(x).float())
-            out = (out.float() + self.shared(x).float() * g).to(x.dtype)
-        return out
+            shared, gate = self.shared(x), self.shared_gate(x)
+        return ops.expert_epilogue(out, x, topw if self.identity else None, topi if self.identity else None,
+                                   self.real_experts, shared, gate)

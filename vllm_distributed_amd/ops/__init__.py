@@ -747,3 +747,11 @@ def latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale: floa
         attention_calls["hip"] += 1
         return _hip.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank, max_seq_len)
     return torch_ref.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank)
+
+
+def expert_epilogue(routed, x, topw, topi, real_experts: int, shared, gate):
+    """What follows the routed experts of a block with identity experts and a gated shared expert, in one pass; see
+    ``torch_ref.expert_epilogue``."""
+    if _use_hip(routed) and (topi is None or topi.dtype == torch.int32):
+        return _hip.expert_epilogue(routed, x, topw, topi, real_experts, shared, gate)
+    return torch_ref.expert_epilogue(routed, x, topw, topi, real_experts, shared, gate)

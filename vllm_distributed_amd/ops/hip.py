@@ -75,6 +75,7 @@ def load() -> ctypes.CDLL:
         "vdamd_gated_rms_norm": [P, P, P, P, L, F, I, I, I, I, P],
         "vdamd_clamped_glu": [P, P, L, I, I, F, F, I, P],
         "vdamd_relu_squared": [P, P, L, I, P],
+        "vdamd_expert_epilogue": [P, P, P, L, P, P, I, I, P, P, L, I, I, I, P],
         "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P],
@@ -1499,4 +1500,25 @@ def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torc
                                            block_table.stride(0), None if token_seq is None else token_seq.data_ptr(),
                                            seq_lens.data_ptr(), float(scale), t, h, dk, rank, cache.shape[2], _dt(q),
                                            _stream()), "latent_row_attention")
+    return out
+
+
+def expert_epilogue(routed: torch.Tensor, x: torch.Tensor, topw: Optional[torch.Tensor], topi: Optional[torch.Tensor],
+                    real_experts: int, shared: Optional[torch.Tensor], gate: Optional[torch.Tensor]) -> torch.Tensor:
+    t, h = routed.shape
+    assert routed.is_contiguous() and x.shape == (t, h) and x.stride(1) == 1 and x.dtype == routed.dtype
+    k = 0
+    if topw is not None:
+        k = topw.shape[1]
+        assert topw.dtype == torch.float32 and topi.dtype == torch.int32 and topw.is_contiguous() and topi.is_contiguous()
+        assert topw.shape == topi.shape == (t, k)
+    if shared is not None:
+        assert shared.shape == (t, h) and shared.is_contiguous() and shared.dtype == routed.dtype
+        assert gate is not None and gate.numel() == t and gate.dtype == routed.dtype
+    out = torch.empty_like(routed)
+    _check(_LIB.vdamd_expert_epilogue(out.data_ptr(), routed.data_ptr(), x.data_ptr(), x.stride(0), _ptr(topw),
+                                      _ptr(topi), k, int(real_experts), _ptr(shared),
+                                      None if shared is None else gate.data_ptr(),
+                                      0 if shared is None else gate.stride(0), t, h, _dt(routed), _stream()),
+           "expert_epilogue")
     return out

@@ -720,3 +720,16 @@ def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torc
         p = torch.softmax(s.masked_fill(mask, float("-inf")), dim=-1)
         res[mine] = torch.einsum("thn,nd->thd", p, keys[:, :rank])
     return res.to(q.dtype)
+
+
+def expert_epilogue(routed: torch.Tensor, x: torch.Tensor, topw: Optional[torch.Tensor], topi: Optional[torch.Tensor],
+                    real_experts: int, shared: Optional[torch.Tensor], gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """``routed + x * s + shared * sigmoid(gate)`` with ``s`` the sum, per row, of the weights ``topw`` whose output
+    ``topi`` is an identity expert (``>= real_experts``); ``gate`` one value per row.  fp32 arithmetic, result in
+    ``routed``'s dtype."""
+    out = routed.float()
+    if topw is not None:
+        out = out + x.float() * (topw.float() * (topi >= real_experts)).sum(-1, keepdim=True)
+    if shared is not None:
+        out = out + shared.float() * torch.sigmoid(gate.float().reshape(-1, 1))
+    return out.to(routed.dtype)
