@@ -7,8 +7,9 @@
 //   add_layer_norm           residual(fp32) += y ; out = layer norm of the sum                         (one launch)
 //   decay_linear_attention   S <- decay[h] S + k v^T ; o = S^T q per head, q / k / v read (through SiLU) from a fused
 //                            projection, S (dim x vdim, fp32) kept per request slot.  A workgroup owns 64 columns of
-//                            one head's S for one sequence, in registers (4 waves x dim/4 rows each), and walks the
-//                            sequence's rows in order: prompt portions and single decoded rows are the same launch
+//                            one head's S for one sequence, in registers (up to 8 waves x dim/8 rows each), and walks
+//                            the sequence's rows in chunks of 16 staged through LDS: prompt portions and single decoded
+//                            rows are the same launch
 //   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g)
 //   clamped_glu              min(g, L) sigmoid(alpha min(g, L)) (clamp(u, -L, L) + 1) over [g | u]
 //   relu_squared             max(x, 0)^2
@@ -176,26 +177,27 @@ __global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ x
 }
 
 // ------------------------------------------------------------------------------------------------ linear attention
-// grid (sequences, heads, column tiles of 64), 256 threads: thread (g = tid / 64, c = tid % 64) owns rows
-// g * R .. g * R + R - 1 of column c of the head's state, in registers.  x rows hold [q (H * dim) | k (H * dim) |
+// grid (sequences, heads, column tiles of 64), G waves: thread (g = tid / 64, c = tid % 64) owns rows
+// g * R .. g * R + R - 1 of column c of the head's state, in registers (G * R >= dim).  x rows hold [q (H * dim) | k (H * dim) |
 // v (H * vdim) | ..].  The sequence's rows are walked in chunks of DLA_CHUNK: q / k (all of the head) and v (this
 // tile's columns) of a chunk are staged in LDS through SiLU, the next chunk's loads are in flight while the current
-// one is computed, and the four row groups' partial outputs of a chunk are summed after one barrier - two barriers
+// one is computed, and the G row groups' partial outputs of a chunk are summed after one barrier - two barriers
 // per chunk whatever its length, so a single decoded row and a long prompt portion are the same launch.
 constexpr int DLA_CHUNK = 16;
 
-template <typename T, int R>
-__global__ __launch_bounds__(256) void decay_linear_attention_kernel(
+template <typename T, int R, int G>
+__global__ __launch_bounds__(64 * G) void decay_linear_attention_kernel(
     float* __restrict__ out, const T* __restrict__ x, long x_stride, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int H, int dim, int vdim, int silu) {
-  constexpr int C = DLA_CHUNK, W = 4 * R;          // W: the key size padded to the four row groups
-  constexpr int NQ = C * W / 256;                  // q (and k) values a thread stages per chunk
-  constexpr int NV = C * 64 / 256;
+  constexpr int C = DLA_CHUNK, W = G * R, TH = 64 * G;   // W: the key size padded to the G row groups
+  constexpr int NQ = C * W / TH;                          // q (and k) values a thread stages per chunk
+  constexpr int NV = C * 64 / TH;
+  static_assert(R % 4 == 0 && (C * W) % TH == 0 && (C * 64) % TH == 0, "chunk does not divide over the threads");
   __shared__ __attribute__((aligned(16))) float qs[C][W];
   __shared__ __attribute__((aligned(16))) float ks[C][W];
   __shared__ float vs[C][64];
-  __shared__ float part[4][C][64];
+  __shared__ float part[G][C][64];
   const int b = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, g = tid >> 6, lane = tid & 63;
   const int col0 = blockIdx.z * 64;
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(256) void decay_linear_attention_kernel(
   auto fetch = [&](int r0) {                       // rows r0 .. of the sequence into registers (zero beyond its end)
 #pragma unroll
     for (int u = 0; u < NQ; ++u) {
-      const int idx = tid + 256 * u, t = idx / W, j = idx - t * W;
+      const int idx = tid + TH * u, t = idx / W, j = idx - t * W;
       const bool ok = r0 + t < e && j < dim;
       const T* xr = x + (long)(r0 + t) * x_stride;
       pq[u] = ok ? act(ldf(xr + qoff + j)) : 0.f;
@@ -225,7 +227,7 @@ __global__ __launch_bounds__(256) void decay_linear_attention_kernel(
     }
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int idx = tid + 256 * u, t = idx >> 6, c = idx & 63;
+      const int idx = tid + TH * u, t = idx >> 6, c = idx & 63;
       const bool ok = r0 + t < e && col0 + c < vdim;
       pv[u] = ok ? act(ldf(x + (long)(r0 + t) * x_stride + voff + c)) : 0.f;
     }
@@ -235,38 +237,42 @@ __global__ __launch_bounds__(256) void decay_linear_attention_kernel(
     const int n = min(C, e - r0);
 #pragma unroll
     for (int u = 0; u < NQ; ++u) {
-      const int idx = tid + 256 * u, t = idx / W, j = idx - t * W;
+      const int idx = tid + TH * u, t = idx / W, j = idx - t * W;
       qs[t][j] = pq[u];
       ks[t][j] = pk[u];
     }
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int idx = tid + 256 * u;
+      const int idx = tid + TH * u;
       vs[idx >> 6][idx & 63] = pv[u];
     }
     if (r0 + C < e) fetch(r0 + C);
     __syncthreads();
+#pragma unroll 2
     for (int t = 0; t < n; ++t) {
       const float v = vs[t][lane];
       const float4* k4 = reinterpret_cast<const float4*>(&ks[t][g * R]);
       const float4* q4 = reinterpret_cast<const float4*>(&qs[t][g * R]);
-      float acc = 0.f;
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;              // (four chains: the sums do not wait for each other)
 #pragma unroll
       for (int i = 0; i < R / 4; ++i) {
         const float4 kk = k4[i], qq = q4[i];
-        S[4 * i] = d * S[4 * i] + kk.x * v;         acc += S[4 * i] * qq.x;
-        S[4 * i + 1] = d * S[4 * i + 1] + kk.y * v; acc += S[4 * i + 1] * qq.y;
-        S[4 * i + 2] = d * S[4 * i + 2] + kk.z * v; acc += S[4 * i + 2] * qq.z;
-        S[4 * i + 3] = d * S[4 * i + 3] + kk.w * v; acc += S[4 * i + 3] * qq.w;
+        S[4 * i] = d * S[4 * i] + kk.x * v;         a0 += S[4 * i] * qq.x;
+        S[4 * i + 1] = d * S[4 * i + 1] + kk.y * v; a1 += S[4 * i + 1] * qq.y;
+        S[4 * i + 2] = d * S[4 * i + 2] + kk.z * v; a2 += S[4 * i + 2] * qq.z;
+        S[4 * i + 3] = d * S[4 * i + 3] + kk.w * v; a3 += S[4 * i + 3] * qq.w;
       }
-      part[g][t][lane] = acc;
+      part[g][t][lane] = (a0 + a1) + (a2 + a3);
     }
     __syncthreads();
-    for (int idx = tid; idx < n * 64; idx += 256) {
+    for (int idx = tid; idx < n * 64; idx += TH) {
       const int t = idx >> 6, c = idx & 63;
-      if (col0 + c < vdim)
-        out[(long)(r0 + t) * H * vdim + (long)h * vdim + col0 + c] =
-            (part[0][t][c] + part[1][t][c]) + (part[2][t][c] + part[3][t][c]);
+      if (col0 + c < vdim) {
+        float sum = 0.f;
+#pragma unroll
+        for (int gg = 0; gg < G; ++gg) sum += part[gg][t][c];
+        out[(long)(r0 + t) * H * vdim + (long)h * vdim + col0 + c] = sum;
+      }
     }
   }
   if (col) {
@@ -540,22 +546,33 @@ VDAMD_API int vdamd_relu_squared(void* out, const void* x, long n, int dt, hipSt
   return 0;
 }
 
-// x [T, x_stride] of type dt, out fp32 [T, H * vdim], state fp32 [slots, H, dim, vdim]; dim <= 256
+// x [T, x_stride] of type dt, out fp32 [T, H * vdim], state fp32 [slots, H, dim, vdim]; dim <= 256.  max_rows: the most
+// rows any sequence brings (0 = unknown)
 VDAMD_API int vdamd_decay_linear_attention(float* out, const void* x, long x_stride, const float* decay, float* state,
                                            const int* slots, const int* qsl, const int* seq_lens, int num_seqs, int H,
-                                           int dim, int vdim, int silu, int dt, hipStream_t stream) {
+                                           int dim, int vdim, int silu, int max_rows, int dt, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
   if (H <= 0 || dim <= 0 || vdim <= 0 || dim > 256) return 1;
   const dim3 grid(num_seqs, H, (vdim + 63) / 64);
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
-#define DLA(R_)                                                                                                      \
-  hipLaunchKernelGGL((decay_linear_attention_kernel<TT, R_>), grid, dim3(256), 0, stream, out, (const TT*)x, x_stride, \
-                     decay, state, slots, qsl, seq_lens, H, dim, vdim, silu)
-    if (dim <= 32) DLA(8);
-    else if (dim <= 64) DLA(16);
-    else if (dim <= 128) DLA(32);
-    else DLA(64);
+#define DLA(R_, G_)                                                                                              \
+  hipLaunchKernelGGL((decay_linear_attention_kernel<TT, R_, G_>), grid, dim3(64 * G_), 0, stream, out, (const TT*)x, \
+                     x_stride, decay, state, slots, qsl, seq_lens, H, dim, vdim, silu)
+    if (max_rows > 0 && max_rows <= 2) {
+      // decoded rows only: the launch is bound by reading and writing the states, so small workgroups, several of
+      // which fit a CU and overlap each other's loads
+      if (dim <= 32) DLA(8, 4);
+      else if (dim <= 64) DLA(16, 4);
+      else if (dim <= 128) DLA(32, 4);
+      else DLA(64, 4);
+    } else {
+      // prompt portions: the walk over the rows is sequential, so as many waves per workgroup as the rows allow
+      if (dim <= 32) DLA(8, 4);
+      else if (dim <= 64) DLA(8, 8);
+      else if (dim <= 128) DLA(8, 16);
+      else DLA(16, 16);
+    }
 #undef DLA
   });
   if (rc) return 1;

@@ -76,7 +76,7 @@ def load() -> ctypes.CDLL:
         "vdamd_clamped_glu": [P, P, L, I, I, F, F, I, P],
         "vdamd_relu_squared": [P, P, L, I, P],
         "vdamd_expert_epilogue": [P, P, P, L, P, P, I, I, P, P, L, I, I, I, P],
-        "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, P],
+        "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P],
     }
@@ -1416,7 +1416,8 @@ def decay_linear_attention(x: torch.Tensor, num_heads: int, dim: int, vdim: int,
     _check(_LIB.vdamd_decay_linear_attention(out.data_ptr(), x.data_ptr(), x.stride(0),
                                              _f32_vec(decay, num_heads, "decay").data_ptr(), state.data_ptr(),
                                              slots.data_ptr(), query_start_loc.data_ptr(), seq_lens.data_ptr(), n,
-                                             num_heads, dim, vdim, int(bool(silu)), _dt(x), _stream()),
+                                             num_heads, dim, vdim, int(bool(silu)), int(max_query_len), _dt(x),
+                                             _stream()),
            "decay_linear_attention")
     return out
 
