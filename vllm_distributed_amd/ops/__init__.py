@@ -705,10 +705,9 @@ def add_layer_norm(y, residual, weight, bias, eps: float, out_dtype):
 
 
 def decay_linear_attention(x, num_heads: int, dim: int, vdim: int, decay, state, slots, query_start_loc, seq_lens,
-                           silu: bool = True, max_query_len: int = 0, token_seq=None):
+                           silu: bool = True, max_query_len: int = 0):
     """Linear attention with a per-head decay and a per-request fp32 state; see
-    ``torch_ref.decay_linear_attention``.  ``max_query_len`` (0: unknown) and ``token_seq`` (the sequence of every
-    row, None: row ``t`` is sequence ``t``) only help the kernels choose their launch."""
+    ``torch_ref.decay_linear_attention``.  ``max_query_len`` (0: unknown) only helps the kernel choose its launch."""
     if _use_hip(x):
         return _hip.decay_linear_attention(x, num_heads, dim, vdim, decay, state, slots, query_start_loc, seq_lens,
                                            silu, max_query_len)
