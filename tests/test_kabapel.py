@@ -240,6 +240,23 @@ def test_prefill_then_long_token_by_token_decoding(name, device, dtype, tol, tmp
     check(got, name, cfg, w, {"r": toks}, tol, dtype)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-4), ("bfloat16", 0.35)])
+@pytest.mark.parametrize("name", ["varied", "fragments"])
+def test_pages_of_64_tokens(name, dtype, tol, tmp_path_factory, tmp_path):
+    """The page size a GPU engine uses by default: two requests in turn, portions that end inside, at and just
+    behind a page's border, then single rows across the next border."""
+    path, cfg, w = model_dir(name, tmp_path_factory, dtype)
+    a, b = tokens_for(cfg, 150, 60), tokens_for(cfg, 70, 61)
+    steps = [[("a", a[:63], [0, 62])], [("a", a[63:64], [0]), ("b", b[:64], [63])], [("a", a[64:66], [0, 1]), ("b", b[64:65], [0])],
+             [("a", a[66:127], [60]), ("b", b[65:70], [4]), {"end": ["b"]}]]
+    steps += [[("a", a[i:i + 1], [0])] for i in range(127, 150)]
+    steps[-1].append({"end": ["a"]})
+    got = run_schedule(path, steps, dtype, "cuda", max_tokens=256, block_size=64, tmp=tmp_path)
+    assert len(got) == 2 + 1 + 1 + 2 + 1 + 1 + 1 + 23
+    check(got, name, cfg, w, {"a": a, "b": b}, tol)
+
+
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
 @pytest.mark.parametrize("sizes", [[2], [3, 2, 7, 1, 16, 17, 2, 2, 31, 5], [1], [64, 2, 1]])
 def test_portions_of_any_size(sizes, device, dtype, tol, tmp_path_factory, tmp_path):
