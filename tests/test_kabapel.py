@@ -80,6 +80,11 @@ CONFIGS = {
     # a latent width the matrix-core kernel is built for (64 + 32): rows and V^T fragments, shared with a reader
     "fragments": config([latent(4, 16, 32, 16, 64, 0.2, rot(32), dense(64)), lightning(2, 32, 32, [0.9, 0.99], dense(48)),
                          latent(3, 8, 32, 24, 64, 0.2, rot(32), moe(4, 1, 2, 32, 1.0), kv_from=0)], width=64),
+    # sizes that are multiples of nothing much: a width the grouped expert kernels do not take (the experts then run
+    # one after the other, also in bfloat16 on the GPU, and decode steps are not captured)
+    "odd": config([lightning(3, 20, 28, [0.6, 0.9, 0.97], moe(5, 1, 2, 12, 1.1, groups=(3, 2), shared=(20, 1.4))),
+                   latent(3, 20, 12, 28, 36, 0.18, rot(12), dense(60)),
+                   latent(5, 12, 12, 4, 36, 0.25, rot(12), moe(3, 0, 3, 28, 0.7), kv_from=1)], width=100, vocab=333),
     # wider, for pages of 16 tokens
     "paged": config([lightning(4, 16, 16, [0.8, 0.95, 0.99, 0.999], dense(96)),
                      latent(4, 16, 8, 16, 32, 0.2, rot(8), moe(6, 2, 2, 32, 1.0, groups=(4, 3), shared=(32, 1.0))),
@@ -229,7 +234,7 @@ def test_residual_stream_after_every_layer(device, dtype, tol, tmp_path_factory)
 
 
 @pytest.mark.parametrize("device,dtype,tol", DEVICES)
-@pytest.mark.parametrize("name", ["varied", "paged", "recurrent_only", "fragments"])
+@pytest.mark.parametrize("name", ["varied", "paged", "recurrent_only", "fragments", "odd"])
 def test_prefill_then_long_token_by_token_decoding(name, device, dtype, tol, tmp_path_factory, tmp_path):
     """A prompt, then 150 tokens one at a time: the state is carried through 150 single-row steps, the cache grows
     over several pages."""
