@@ -7,9 +7,9 @@
 //   add_layer_norm           residual(fp32) += y ; out = layer norm of the sum                         (one launch)
 //   decay_linear_attention   S <- decay[h] S + k v^T ; o = S^T q per head, q / k / v read (through SiLU) from a fused
 //                            projection, S (dim x vdim, fp32) kept per request slot.  A workgroup owns 64 columns of
-//                            one head's S for one sequence, in registers (up to 8 waves x dim/8 rows each), and walks
-//                            the sequence's rows in chunks of 16 staged through LDS: prompt portions and single decoded
-//                            rows are the same launch
+//                            one head's S for one sequence, in registers (up to 16 waves x dim/16 rows each), and walks
+//                            the sequence's rows in chunks staged through LDS: prompt portions and single decoded rows
+//                            are the same kernel (launches of decoded rows only take small workgroups)
 //   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g)
 //   clamped_glu              min(g, L) sigmoid(alpha min(g, L)) (clamp(u, -L, L) + 1) over [g | u]
 //   relu_squared             max(x, 0)^2
@@ -179,21 +179,19 @@ __global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ x
 // ------------------------------------------------------------------------------------------------ linear attention
 // grid (sequences, heads, column tiles of 64), G waves: thread (g = tid / 64, c = tid % 64) owns rows
 // g * R .. g * R + R - 1 of column c of the head's state, in registers (G * R >= dim).  x rows hold [q (H * dim) | k (H * dim) |
-// v (H * vdim) | ..].  The sequence's rows are walked in chunks of DLA_CHUNK: q / k (all of the head) and v (this
+// v (H * vdim) | ..].  The sequence's rows are walked in chunks of C: q / k (all of the head) and v (this
 // tile's columns) of a chunk are staged in LDS through SiLU, the next chunk's loads are in flight while the current
 // one is computed, and the G row groups' partial outputs of a chunk are summed after one barrier - two barriers
 // per chunk whatever its length, so a single decoded row and a long prompt portion are the same launch.
-constexpr int DLA_CHUNK = 16;
-
-template <typename T, int R, int G>
-__global__ __launch_bounds__(64 * G) void decay_linear_attention_kernel(
+template <typename T, int R, int G, int C>
+__global__ __launch_bounds__(64 * G) __attribute__((amdgpu_waves_per_eu(G >= 16 ? 8 : 1, 8))) void decay_linear_attention_kernel(
     float* __restrict__ out, const T* __restrict__ x, long x_stride, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int H, int dim, int vdim, int silu) {
-  constexpr int C = DLA_CHUNK, W = G * R, TH = 64 * G;   // W: the key size padded to the G row groups
+  constexpr int W = G * R, TH = 64 * G;                   // W: the key size padded to the G row groups
   constexpr int NQ = C * W / TH;                          // q (and k) values a thread stages per chunk
-  constexpr int NV = C * 64 / TH;
-  static_assert(R % 4 == 0 && (C * W) % TH == 0 && (C * 64) % TH == 0, "chunk does not divide over the threads");
+  constexpr int NV = (C * 64 + TH - 1) / TH;              // (with more threads than v values, the first ones stage)
+  static_assert(R % 4 == 0 && (C * W) % TH == 0, "chunk does not divide over the threads");
   __shared__ __attribute__((aligned(16))) float qs[C][W];
   __shared__ __attribute__((aligned(16))) float ks[C][W];
   __shared__ float vs[C][64];
@@ -228,7 +226,7 @@ __global__ __launch_bounds__(64 * G) void decay_linear_attention_kernel(
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + TH * u, t = idx >> 6, c = idx & 63;
-      const bool ok = r0 + t < e && col0 + c < vdim;
+      const bool ok = idx < C * 64 && r0 + t < e && col0 + c < vdim;
       pv[u] = ok ? act(ldf(x + (long)(r0 + t) * x_stride + voff + c)) : 0.f;
     }
   };
@@ -244,7 +242,7 @@ __global__ __launch_bounds__(64 * G) void decay_linear_attention_kernel(
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + TH * u;
-      vs[idx >> 6][idx & 63] = pv[u];
+      if (idx < C * 64) vs[idx >> 6][idx & 63] = pv[u];
     }
     if (r0 + C < e) fetch(r0 + C);
     __syncthreads();
@@ -556,22 +554,22 @@ VDAMD_API int vdamd_decay_linear_attention(float* out, const void* x, long x_str
   const dim3 grid(num_seqs, H, (vdim + 63) / 64);
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
-#define DLA(R_, G_)                                                                                              \
-  hipLaunchKernelGGL((decay_linear_attention_kernel<TT, R_, G_>), grid, dim3(64 * G_), 0, stream, out, (const TT*)x, \
-                     x_stride, decay, state, slots, qsl, seq_lens, H, dim, vdim, silu)
+#define DLA(R_, G_, C_)                                                                                          \
+  hipLaunchKernelGGL((decay_linear_attention_kernel<TT, R_, G_, C_>), grid, dim3(64 * G_), 0, stream, out,          \
+                     (const TT*)x, x_stride, decay, state, slots, qsl, seq_lens, H, dim, vdim, silu)
     if (max_rows > 0 && max_rows <= 2) {
       // decoded rows only: the launch is bound by reading and writing the states, so small workgroups, several of
       // which fit a CU and overlap each other's loads
-      if (dim <= 32) DLA(8, 4);
-      else if (dim <= 64) DLA(16, 4);
-      else if (dim <= 128) DLA(32, 4);
-      else DLA(64, 4);
+      if (dim <= 32) DLA(8, 4, 8);
+      else if (dim <= 64) DLA(16, 4, 4);
+      else if (dim <= 128) DLA(32, 4, 4);
+      else DLA(64, 4, 4);
     } else {
       // prompt portions: the walk over the rows is sequential, so as many waves per workgroup as the rows allow
-      if (dim <= 32) DLA(8, 4);
-      else if (dim <= 64) DLA(8, 8);
-      else if (dim <= 128) DLA(8, 16);
-      else DLA(16, 16);
+      if (dim <= 32) DLA(8, 4, 8);
+      else if (dim <= 64) DLA(8, 8, 8);
+      else if (dim <= 128) DLA(8, 16, 8);
+      else DLA(16, 16, 8);
     }
 #undef DLA
   });
