@@ -39,6 +39,8 @@ template <typename F> int by_dtype(int dt, F&& f) {
 
 int row_threads(int h) { return h >= 2048 ? 512 : (h >= 512 ? 256 : 128); }
 
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 template <typename T>
@@ -97,6 +99,36 @@ __global__ void gated_rms_norm_kernel(TO* __restrict__ out, const float* __restr
   for (int i = threadIdx.x; i < N; i += blockDim.x) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)));
 }
 
+// 16-bit gate and result, rows whose length and gate stride are multiples of 8: 16-byte accesses
+template <typename T>
+__global__ void gated_rms_norm_vec_kernel(T* __restrict__ out, const float* __restrict__ o, const float* __restrict__ w,
+                                          const T* __restrict__ gate, long gate_stride, float eps, int N) {
+  using V8 = typename Vec8<T>::type;
+  __shared__ float red[17];
+  const long row = blockIdx.x;
+  const float4* o4 = reinterpret_cast<const float4*>(o + row * (long)N);
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+  const T* g = gate + row * gate_stride;
+  const int nv = N >> 3;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const float4 a = o4[2 * i], b = o4[2 * i + 1];
+    ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)N + eps);
+  T* dst = out + row * (long)N;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const float4 a = o4[2 * i], b = o4[2 * i + 1], wa = w4[2 * i], wb = w4[2 * i + 1];
+    const V8 gv = ld8<T>(g + 8 * i);
+    const float of[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    const float wf[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    V8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (T)(of[e] * inv * wf[e] * sigmoid_f((float)gv[e]));
+    st8<T>(dst + 8 * i, r);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ activations
 template <typename T>
 __global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ h, long h_stride, int F, float limit,
@@ -138,7 +170,7 @@ template <typename T>
 __global__ void expert_epilogue_kernel(T* __restrict__ out, const T* __restrict__ routed, const T* __restrict__ x,
                                        long x_stride, const float* __restrict__ topw, const int* __restrict__ topi,
                                        int k, int real_experts, const T* __restrict__ shared,
-                                       const T* __restrict__ gate, long gate_stride, int H) {
+                                       const T* __restrict__ gate, long gate_stride, int H, bool vec) {
   const long row = blockIdx.x;
   float share = 0.f;
   if (topw != nullptr)
@@ -150,7 +182,7 @@ __global__ void expert_epilogue_kernel(T* __restrict__ out, const T* __restrict_
   const T* sr = shared != nullptr ? shared + row * (long)H : nullptr;
   T* o = out + row * (long)H;
   if constexpr (!std::is_same_v<T, float>) {
-    if ((H & 7) == 0 && (x_stride & 7) == 0) {
+    if (vec) {
       using V8 = typename Vec8<T>::type;
       for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
         const V8 rv = ld8<T>(rr + i), xv = ld8<T>(xr + i);
@@ -480,6 +512,18 @@ VDAMD_API int vdamd_gated_rms_norm(void* out, const float* o, const float* w, co
   if (rows <= 0) return 0;
   if (N <= 0) return 1;
   int inner = 0;
+  if (gate_dt != DT_F32 && gate_dt == out_dt && N % 8 == 0 && gate_stride % 8 == 0 && aligned16(gate) && aligned16(o) &&
+      aligned16(w) && aligned16(out)) {
+    const int rv = by_dtype(gate_dt, [&](auto* tg) {
+      using TG = std::remove_pointer_t<decltype(tg)>;
+      if constexpr (!std::is_same_v<TG, float>)
+        hipLaunchKernelGGL((gated_rms_norm_vec_kernel<TG>), dim3(rows), dim3(N >= 2048 ? 256 : 128), 0, stream, (TG*)out,
+                           o, w, (const TG*)gate, gate_stride, eps, N);
+    });
+    if (rv) return 1;
+    HIP_LAUNCH_CHECK();
+    return 0;
+  }
   const int rc = by_dtype(gate_dt, [&](auto* tg) {
     using TG = std::remove_pointer_t<decltype(tg)>;
     inner = by_dtype(out_dt, [&](auto* to) {
@@ -500,7 +544,7 @@ VDAMD_API int vdamd_clamped_glu(void* out, const void* h, long h_stride, int row
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
     if constexpr (!std::is_same_v<TT, float>) {
-      if (F % 8 == 0 && h_stride % 8 == 0) {
+      if (F % 8 == 0 && h_stride % 8 == 0 && aligned16(h) && aligned16(out)) {
         hipLaunchKernelGGL((clamped_glu_vec_kernel<TT>), dim3(rows, (F + 2047) / 2048), dim3(256), 0, stream, (TT*)out,
                            (const TT*)h, h_stride, F, limit, alpha);
         return;
@@ -521,11 +565,14 @@ VDAMD_API int vdamd_expert_epilogue(void* out, const void* routed, const void* x
                                     long gate_stride, int rows, int H, int dt, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H <= 0 || (topw != nullptr && (topi == nullptr || k < 1)) || (shared != nullptr && gate == nullptr)) return 1;
+  // 16-byte accesses where every row of every operand starts on a 16-byte border
+  const bool vec = H % 8 == 0 && x_stride % 8 == 0 && aligned16(out) && aligned16(routed) && aligned16(x) &&
+                   (shared == nullptr || aligned16(shared));
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
     hipLaunchKernelGGL((expert_epilogue_kernel<TT>), dim3(rows), dim3(H >= 2048 ? 256 : 128), 0, stream, (TT*)out,
                        (const TT*)routed, (const TT*)x, x_stride, topw, topi, k, real_experts, (const TT*)shared,
-                       (const TT*)gate, gate_stride, H);
+                       (const TT*)gate, gate_stride, H, vec);
   });
   if (rc) return 1;
   HIP_LAUNCH_CHECK();
